@@ -41,13 +41,23 @@ def _load_builtin() -> None:
 def architecture_of(config: Mapping) -> Architecture:
     """The registered architecture a config.json dict names."""
     _load_builtin()
-    names = config.get("architectures")
-    if not isinstance(names, (list, tuple)) or not names or not isinstance(names[0], str):
-        raise ConfigError("missing/invalid config key: architectures (want a list with the model class name)")
-    arch = _ARCHITECTURES.get(names[0])
+    name = architecture_name(config)
+    arch = _ARCHITECTURES.get(name)
     if arch is None:
-        raise ConfigError(f"unknown architecture: {names[0]} (registered: {', '.join(sorted(_ARCHITECTURES))})")
+        raise ConfigError(f"unknown architecture: {name} (registered: {', '.join(sorted(_ARCHITECTURES))})")
     return arch
+
+
+def architecture_name(config: Mapping) -> str:
+    """The name a config.json dict gives its model class: the first of ``architectures`` (a list),
+    or, in files that name one class only, the string under ``architecture``."""
+    names = config.get("architectures")
+    if names is None and isinstance(config.get("architecture"), str):
+        return config["architecture"]
+    if not isinstance(names, (list, tuple)) or not names or not isinstance(names[0], str):
+        raise ConfigError("missing/invalid config key: architectures (want a list with the model class name, "
+                          "or a string under 'architecture')")
+    return names[0]
 
 
 def load_config(folder: str):

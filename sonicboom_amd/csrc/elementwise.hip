@@ -87,6 +87,69 @@ extern "C" int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype,
   return sb::check_launch("sb_cast");
 }
 
+// ---- a scaled residual add, and activations of an ungated feed-forward ------------------------
+namespace {
+
+template <typename TI>
+__global__ void add_scaled_kernel(float *__restrict__ resid, const TI *__restrict__ y, float scale, size_t n) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx < n) resid[idx] = ld_f(y, idx) * scale + resid[idx];
+}
+
+__device__ __forceinline__ float softplus_f(float a) { return a > 20.0f ? a : log1pf(expf(a)); }
+
+// xIELU with the two numbers (p, q) of a layer: for z > 0 softplus(p) z^2 + z/2, else
+// (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2.
+template <typename TO, typename TI>
+__global__ void activate_kernel(TO *__restrict__ out, const TI *__restrict__ in, size_t n, int kind,
+                                const void *__restrict__ params, int params_dtype) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const float z = ld_f(in, idx);
+  float v;
+  if (kind == SB_ACT_XIELU) {
+    const float ap = softplus_f(ld_dyn(params, params_dtype, 0));
+    const float an = 0.5f + softplus_f(ld_dyn(params, params_dtype, 1));
+    v = z > 0.0f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z;
+  } else {
+    v = gate_act(z, kind == SB_ACT_GELU_TANH ? SB_GATE_GELU_TANH : SB_GATE_SILU);
+  }
+  st_f(out, idx, v);
+}
+
+}  // namespace
+
+extern "C" int sb_add_scaled(float *resid, const void *y, int y_dtype, float scale, size_t n, void *stream) {
+  SB_REQUIRE(resid && y, "sb_add_scaled: null pointer");
+  SB_REQUIRE(sb::valid_dtype(y_dtype), "sb_add_scaled: unknown dtype");
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(n, 256);
+  if (y_dtype == SB_F32) add_scaled_kernel<float><<<nb, 256, 0, s>>>(resid, (const float *)y, scale, n);
+  else add_scaled_kernel<bf16_t><<<nb, 256, 0, s>>>(resid, (const bf16_t *)y, scale, n);
+  return sb::check_launch("sb_add_scaled");
+}
+
+extern "C" int sb_activate(void *out, int out_dtype, const void *in, int in_dtype, size_t n, int kind,
+                           const void *params, int params_dtype, void *stream) {
+  SB_REQUIRE(out && in, "sb_activate: null pointer");
+  SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(in_dtype), "sb_activate: unknown dtype");
+  SB_SUPPORT(kind == SB_ACT_SILU || kind == SB_ACT_GELU_TANH || kind == SB_ACT_XIELU,
+             "sb_activate: unknown activation %d", kind);
+  SB_REQUIRE(kind != SB_ACT_XIELU || (params && sb::valid_dtype(params_dtype)),
+             "sb_activate: xIELU needs its two numbers");
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(n, 256);
+#define SB_GO(TO, TI) activate_kernel<TO, TI><<<nb, 256, 0, s>>>((TO *)out, (const TI *)in, n, kind, params, params_dtype)
+  if (out_dtype == SB_F32 && in_dtype == SB_F32) SB_GO(float, float);
+  else if (out_dtype == SB_BF16 && in_dtype == SB_F32) SB_GO(bf16_t, float);
+  else if (out_dtype == SB_BF16 && in_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
+  else SB_GO(float, bf16_t);
+#undef SB_GO
+  return sb::check_launch("sb_activate");
+}
+
 // ---- measurement: how fast can this GPU stream memory? ---------------------------------------
 namespace {
 __global__ void __launch_bounds__(256)

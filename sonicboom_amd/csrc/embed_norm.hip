@@ -186,7 +186,116 @@ reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float 
   }
 }
 
+
+// RMS norm in groups: the row is cut into `groups` equal consecutive parts and each is divided by
+// its own sqrt(mean(part^2) + eps); the weight spans the row.  With `partial` the row is first
+// updated, x[t,:] += scale * (sum of the slices in ascending order + bias).  One block of four
+// waves per row.  A group belongs to one wave, or, when the row has fewer groups than the block has
+// waves, to 4 / groups waves that take every such share of its elements and meet in LDS; the sums
+// of squares are double and their order depends on the row's width and groups alone, so a row's
+// result has the same bits whatever else the launch holds.
+constexpr int kGroupThreads = 256;
+constexpr int kGroupWaves = kGroupThreads / 64;
+
+template <typename TO>
+__global__ void __launch_bounds__(kGroupThreads)
+group_norm_kernel(TO *__restrict__ y, float *x, const int32_t *__restrict__ rows,
+                  const float *__restrict__ partial, int n_slices, size_t slice_stride,
+                  const void *__restrict__ bias, int bias_dtype, float scale, const void *__restrict__ w,
+                  int w_dtype, int width, int groups, float eps, int do_norm) {
+  __shared__ double wave_part[kGroupWaves];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float *xr = x + size_t(src) * width;
+  const float *pr = partial ? partial + size_t(r) * width : nullptr;
+  TO *yr = y + size_t(r) * width;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int gw = width / groups;
+  const int wpg = groups >= kGroupWaves ? 1 : kGroupWaves / groups;   // waves that share a group: 1, 2 or 4
+  const int per_pass = kGroupWaves / wpg;                              // groups the block takes at a time
+  for (int g0 = 0; g0 < groups; g0 += per_pass) {
+    const int g = g0 + wave / wpg, k = wave % wpg;
+    const bool active = g < groups;
+    double part = 0.0;
+    if (active) {
+      for (int i = lane + 64 * k; i < gw; i += 64 * wpg) {
+        const size_t e = size_t(g) * gw + i;
+        float v;
+        if (pr) {
+          float acc = pr[e];
+          for (int s = 1; s < n_slices; ++s) acc += pr[size_t(s) * slice_stride + e];
+          if (bias) acc += ld_dyn(bias, bias_dtype, e);
+          v = acc * scale + xr[e];
+          xr[e] = v;
+        } else {
+          v = xr[e];
+        }
+        part += double(v * v);
+      }
+      part = wave_sum(part);
+      if (lane == 0) wave_part[wave] = part;
+    }
+    if (!do_norm) continue;
+    __syncthreads();
+    if (active) {
+      double total = 0.0;
+      for (int j = 0; j < wpg; ++j) total += wave_part[(wave / wpg) * wpg + j];
+      const float inv = 1.0f / sqrtf(float(total / double(gw)) + eps);
+      for (int i = lane + 64 * k; i < gw; i += 64 * wpg) {
+        const size_t e = size_t(g) * gw + i;
+        float o = xr[e] * inv;
+        if (w) o = o * ld_dyn(w, w_dtype, e);
+        st_f(yr, e, o);
+      }
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
+
+// y[r,:] = RMS norm of x[src,:] in `groups` equal consecutive parts, times w (see group_norm_kernel).
+extern "C" int sb_rmsnorm_grouped(void *y, int out_dtype, const float *x, const void *w, int w_dtype,
+                                  const int32_t *rows, int n_rows, int width, int groups, float eps, void *stream) {
+  SB_REQUIRE(y && x, "sb_rmsnorm_grouped: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && groups > 0, "sb_rmsnorm_grouped: bad sizes rows=%d width=%d groups=%d",
+             n_rows, width, groups);
+  SB_REQUIRE(width % groups == 0, "sb_rmsnorm_grouped: %d groups do not divide a row of %d", groups, width);
+  SB_REQUIRE(sb::valid_dtype(out_dtype) && (!w || sb::valid_dtype(w_dtype)), "sb_rmsnorm_grouped: unknown dtype");
+  SB_REQUIRE(eps >= 0.0f, "sb_rmsnorm_grouped: eps must not be negative");
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == SB_F32)
+    group_norm_kernel<float><<<n_rows, kGroupThreads, 0, s>>>((float *)y, const_cast<float *>(x), rows, nullptr, 0, 0,
+                                                              nullptr, 0, 1.0f, w, w_dtype, width, groups, eps, 1);
+  else
+    group_norm_kernel<bf16_t><<<n_rows, kGroupThreads, 0, s>>>((bf16_t *)y, const_cast<float *>(x), rows, nullptr, 0, 0,
+                                                               nullptr, 0, 1.0f, w, w_dtype, width, groups, eps, 1);
+  return sb::check_launch("sb_rmsnorm_grouped");
+}
+
+// x[t,:] += scale * (sum over slices of partial[s][t][:] (+ bias)); with do_norm also
+// y[t,:] = the RMS norm of x[t,:] in `groups` parts, times w, in y_dtype.  Any width.
+extern "C" int sb_reduce_scaled_group_norm(void *y, int y_dtype, float *x, const float *partial, int n_slices,
+                                           const void *bias, int bias_dtype, float scale, const void *w, int w_dtype,
+                                           int n_rows, int width, int groups, float eps, int do_norm, void *stream) {
+  SB_REQUIRE(x && partial && (!do_norm || y), "sb_reduce_scaled_group_norm: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && n_slices >= 1 && groups > 0, "sb_reduce_scaled_group_norm: bad sizes");
+  SB_REQUIRE(width % groups == 0, "sb_reduce_scaled_group_norm: %d groups do not divide a row of %d", groups, width);
+  SB_REQUIRE((!do_norm || sb::valid_dtype(y_dtype)) && (!bias || sb::valid_dtype(bias_dtype)) &&
+                 (!w || sb::valid_dtype(w_dtype)),
+             "sb_reduce_scaled_group_norm: unknown dtype");
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t stride = size_t(n_rows) * width;
+  if (!do_norm || y_dtype == SB_F32)
+    group_norm_kernel<float><<<n_rows, kGroupThreads, 0, s>>>((float *)y, x, nullptr, partial, n_slices, stride, bias,
+                                                              bias_dtype, scale, w, w_dtype, width, groups, eps, do_norm);
+  else
+    group_norm_kernel<bf16_t><<<n_rows, kGroupThreads, 0, s>>>((bf16_t *)y, x, nullptr, partial, n_slices, stride, bias,
+                                                               bias_dtype, scale, w, w_dtype, width, groups, eps, do_norm);
+  return sb::check_launch("sb_reduce_scaled_group_norm");
+}
 
 // The widest row sb_reduce_resid_norm takes.
 extern "C" int sb_reduce_resid_norm_max_width(void) { return 4 * kNormKeep * kNormThreads; }

@@ -73,6 +73,10 @@ typedef enum sb_dtype { SB_F32 = 0, SB_BF16 = 1 } sb_dtype;
  * gate in Y = act(X Wg^T) * (X Wu^T). */
 typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2 } sb_gate;
 
+/* The `kind` argument of sb_activate.  xIELU takes two numbers (p, q) from memory: for z > 0
+ * softplus(p) z^2 + z/2, else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */
+typedef enum sb_act { SB_ACT_SILU = 1, SB_ACT_GELU_TANH = 2, SB_ACT_XIELU = 3 } sb_act;
+
 /* Message of this thread's last failed call ("" if none). Never NULL. */
 const char *sb_last_error(void);
 /* A JSON object naming the target architecture, the page size and the build flags. */
@@ -86,6 +90,17 @@ int sb_embed(float *out, const void *table, int table_dtype, const int32_t *ids,
  * x is f32; y is out_dtype; w is w_dtype (NULL = no weight). */
 int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w, int w_dtype,
                const int32_t *rows, int n_rows, int width, float eps, void *stream);
+
+/* The same norm taken over each of `groups` equal consecutive parts of the row (the weight spans
+ * the row); a row's bits do not depend on what else the launch holds. */
+int sb_rmsnorm_grouped(void *y, int out_dtype, const float *x, const void *w, int w_dtype,
+                       const int32_t *rows, int n_rows, int width, int groups, float eps, void *stream);
+
+/* x[t,:] += scale * (sum_s partial[s][t][:] (+ bias)), slices in ascending order; with do_norm also
+ * y[t,:] = the RMS norm of x[t,:] in `groups` parts, times w.  Any width that `groups` divides. */
+int sb_reduce_scaled_group_norm(void *y, int y_dtype, float *x, const float *partial, int n_slices,
+                                const void *bias, int bias_dtype, float scale, const void *w, int w_dtype,
+                                int n_rows, int width, int groups, float eps, int do_norm, void *stream);
 
 /* x[t,:] += sum_s partial[s][t][:] (+ bias), slices in ascending order; with do_norm
  * also y[t,:] = rmsnorm(x[t,:]) * w.  partial is f32 [n_slices][n_rows][width]. */
@@ -110,6 +125,14 @@ int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype,
 
 /* resid[i] += y[i]  (resid f32, y of y_dtype). */
 int sb_add_into(float *resid, const void *y, int y_dtype, size_t n, void *stream);
+
+/* resid[i] += scale * y[i]  (resid f32, y of y_dtype). */
+int sb_add_scaled(float *resid, const void *y, int y_dtype, float scale, size_t n, void *stream);
+
+/* out[i] = act(in[i]), act an sb_act; params: the activation's numbers in memory (xIELU: two), of
+ * params_dtype, NULL for the others. */
+int sb_activate(void *out, int out_dtype, const void *in, int in_dtype, size_t n, int kind,
+                const void *params, int params_dtype, void *stream);
 
 /* dst[i] = src[i] converted. */
 int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n, void *stream);
@@ -146,6 +169,49 @@ int sb_attention(void *out, const void *q, int act_dtype, int q_stride, const vo
                  const void *v_cache, int cache_dtype, const int32_t *page_table, int max_pages,
                  int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows,
                  int heads_q, int heads_kv, int head_dim, float scale, int window, void *stream);
+
+/* ---- a gated recurrence (csrc/recurrent.hip) -------------------------------------------------
+ * minGRU over the rows of a step, sequence by sequence: from p f32 [n_rows, 3 * width] = the
+ * pre-activations (a | u | g) of every row, z = sigmoid(a), cand = u + 1/2 (u >= 0) or sigmoid(u),
+ * S = (1 - z) S + z cand, out[r,:] = S * silu(g); S of sequence s lives in state[slots[s]] (f32
+ * [*, width]) and is left moved on.  chunks NULL: a thread a channel walks the rows in order.  Else
+ * the rows in chunks of at most sb_mingru_chunk_rows() rows of one sequence, int32 [n_chunks, 4]
+ * (first row, rows, sequence, 0) in row order, are folded in parallel, carried serially and walked in
+ * parallel; folded: scratch of 2 * n_chunks * width floats. */
+int sb_mingru_chunk_rows(void);
+int sb_mingru_scan(void *out, int out_dtype, const float *p, float *state, const int32_t *cu_rows,
+                   const int32_t *slots, int n_seqs, int n_rows, int width, const int32_t *chunks,
+                   int n_chunks, float *folded, void *stream);
+
+/* ---- latent attention (csrc/attention_latent.hip) --------------------------------------------
+ * A layer keeps a row [c | r] per token (c: rank numbers, r: rot_dim rotated numbers shared by the
+ * heads) in cache [pages][SB_PAGE][rank + rot_dim]; attention runs in the latent's space.
+ * sb_latent_prepare: from a step's input-product rows p f32 [n_rows, row_stride]: queries at
+ * q_off (head = [dim plain | rot_dim rotated]) -> q_plain [n_rows, heads, dim] and the rotated
+ * parts behind the first rank numbers of q_latent [n_rows, heads, rank + rot_dim]; at kv_off (-1:
+ * nothing is stored) rank numbers RMS-normed with c_weight and eps, and rot_dim rotated, stored
+ * at the row's position.  The first rot_dims of rot_dim numbers turn, pair j by float(pos) *
+ * inv_freq[j]; pairs (2j, 2j+1) when interleaved, else (j, j + rot_dims/2). */
+int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride,
+                      int q_off, int kv_off, const void *c_weight, int c_w_dtype, float eps,
+                      const float *inv_freq, int rot_dims, int interleaved, const int32_t *row_pos,
+                      const int32_t *row_seq, void *cache, int cache_dtype, const int32_t *page_table,
+                      int max_pages, int n_pages_total, int n_rows, int heads, int dim, int rot_dim,
+                      int rank, void *stream);
+/* out[t, a, o] = sum_i in[t, a, i] W[a][i][o], W [heads, n_in, n_out]; (t, a, .) of out at
+ * t * out_stride + a * out_hstride, of in at t * in_stride + a * in_hstride; gate f32 or NULL:
+ * times sigmoid(gate[t * gate_stride + a * n_out + o]). */
+int sb_head_product(void *out, int out_dtype, int out_stride, int out_hstride, const void *in,
+                    int in_dtype, int in_stride, int in_hstride, const void *w, int w_dtype,
+                    const float *gate, int gate_stride, int n_rows, int heads, int n_in, int n_out,
+                    void *stream);
+/* out [n_rows, heads, rank]: for every row and head the softmax-weighted sum of the first rank
+ * numbers of the cached rows j it sees (j <= p, and p - j < window unless window is 0), scores
+ * scale * (q . row); q [n_rows, heads, rank + rot_dim].  One wave per (row, head). */
+int sb_latent_attention(void *out, const void *q, int act_dtype, const void *cache, int cache_dtype,
+                        const int32_t *page_table, int max_pages, int n_pages_total,
+                        const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads, int rank,
+                        int rot_dim, float scale, int window, void *stream);
 
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts

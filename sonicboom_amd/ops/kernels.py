@@ -94,8 +94,9 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
 
 
 def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
-            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """RMS norm of float32 rows ``x`` [n, width]; ``rows`` (int32) picks and orders source rows."""
+            rows: Optional[torch.Tensor] = None, groups: int = 1) -> torch.Tensor:
+    """RMS norm of float32 rows ``x`` [n, width]; ``rows`` (int32) picks and orders source rows;
+    ``groups`` > 1: each of that many equal consecutive parts of a row by its own root mean square."""
     _dev(x, weight, rows)
     if x.dtype != torch.float32 or x.dim() != 2:
         raise KernelLibraryError("rmsnorm input must be float32 [rows, width]")
@@ -107,6 +108,12 @@ def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dty
         _i32(rows, n, "row index")
     y = torch.empty((n, width), dtype=out_dtype, device=x.device)
     lib = library.core()
+    if groups != 1:
+        if groups < 1 or width % groups:
+            raise KernelLibraryError(f"{groups} groups do not divide a row of {width}")
+        check(lib.sb_rmsnorm_grouped(_p(y), _dt(y), _p(x), _p(weight), _dt(weight) if weight is not None else 0,
+                                     _p(rows), n, width, int(groups), float(eps), _stream()))
+        return y
     check(lib.sb_rmsnorm(_p(y), _dt(y), _p(x), _p(weight), _dt(weight) if weight is not None else 0,
                          _p(rows), n, width, float(eps), _stream()))
     return y
@@ -173,6 +180,33 @@ def add_into(resid: torch.Tensor, y: torch.Tensor) -> None:
         raise KernelLibraryError("add_into needs a float32 residual and an addend of the same size")
     lib = library.core()
     check(lib.sb_add_into(_p(resid), _p(y), _dt(y), resid.numel(), _stream()))
+
+
+def add_scaled(resid: torch.Tensor, y: torch.Tensor, scale: float) -> None:
+    """resid += scale * y (float32 residual stream, in place)."""
+    _dev(resid, y)
+    if resid.dtype != torch.float32 or resid.numel() != y.numel():
+        raise KernelLibraryError("add_scaled needs a float32 residual and an addend of the same size")
+    check(library.core().sb_add_scaled(_p(resid), _p(y), _dt(y), float(scale), resid.numel(), _stream()))
+
+
+ACTIVATIONS = {"silu": 1, "gelu_tanh": 2, "xielu": 3}      # sb_act of csrc/sb_hip.h
+
+
+def activate(x: torch.Tensor, out_dtype: torch.dtype, activation: str, params: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """act(x) element by element; ``params``: the numbers an activation reads from memory (xIELU's
+    two, of which the kernel takes the softplus itself)."""
+    _dev(x, params)
+    try:
+        kind = ACTIVATIONS[activation]
+    except KeyError:
+        raise KernelLibraryError(f"unknown activation {activation!r}; known: {sorted(ACTIVATIONS)}") from None
+    if activation == "xielu" and (params is None or params.numel() != 2):
+        raise KernelLibraryError("xIELU takes two numbers")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    check(library.core().sb_activate(_p(out), _dt(out), _p(x), _dt(x), x.numel(), kind, _p(params),
+                                     _dt(params) if params is not None else 0, _stream()))
+    return out
 
 
 def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -448,10 +482,11 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
 
 
 def reduce_resid_norm(partial: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor,
-                      norm_weight: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype]
-                      ) -> Optional[torch.Tensor]:
-    """x += sum of the slices of ``partial`` [slices, rows, width] (+ bias); when ``out_dtype`` is
-    given also returns rmsnorm(x) * norm_weight in that type.  One pass over the row."""
+                      norm_weight: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype],
+                      scale: float = 1.0, groups: int = 1) -> Optional[torch.Tensor]:
+    """x += scale * (sum of the slices of ``partial`` [slices, rows, width] (+ bias)); when
+    ``out_dtype`` is given also returns rmsnorm(x) * norm_weight in that type, the norm taken in
+    ``groups`` parts of the row.  One pass over the row."""
     _dev(partial, bias, x, norm_weight)
     if partial.dim() != 3 or partial.dtype != torch.float32 or x.dtype != torch.float32 \
             or tuple(x.shape) != tuple(partial.shape[1:]):
@@ -462,10 +497,19 @@ def reduce_resid_norm(partial: torch.Tensor, bias: Optional[torch.Tensor], x: to
     if norm_weight is not None and norm_weight.numel() != width:
         raise KernelLibraryError("norm weight does not match the row width")
     lib = library.core()
+    y = torch.empty((t, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    if scale != 1.0 or groups != 1:
+        if groups < 1 or width % groups:
+            raise KernelLibraryError(f"{groups} groups do not divide a row of {width}")
+        check(lib.sb_reduce_scaled_group_norm(
+            _p(y), _dt(y) if y is not None else 0, _p(x), _p(partial), s_, _p(bias),
+            _dt(bias) if bias is not None else 0, float(scale), _p(norm_weight),
+            _dt(norm_weight) if norm_weight is not None else 0, t, width, int(groups), float(eps),
+            1 if out_dtype is not None else 0, _stream()))
+        return y
     if width % 4 or width > lib.sb_reduce_resid_norm_max_width():
         raise KernelLibraryError(f"reduce_resid_norm takes widths in steps of 4 up to "
                                  f"{lib.sb_reduce_resid_norm_max_width()}, not {width}")
-    y = torch.empty((t, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
     check(lib.sb_reduce_resid_norm(_p(y), _dt(y) if y is not None else 0, _p(x), _p(partial), s_, _p(bias),
                                    _dt(bias) if bias is not None else 0, _p(norm_weight),
                                    _dt(norm_weight) if norm_weight is not None else 0, t, width, float(eps),
@@ -473,7 +517,9 @@ def reduce_resid_norm(partial: torch.Tensor, bias: Optional[torch.Tensor], x: to
     return y
 
 
-def reduce_resid_norm_ok(width: int) -> bool:
+def reduce_resid_norm_ok(width: int, scale: float = 1.0, groups: int = 1) -> bool:
+    if scale != 1.0 or groups != 1:
+        return groups >= 1 and width % groups == 0       # the kernel for scaled sums and grouped norms: any width
     return width % 4 == 0 and width <= library.core().sb_reduce_resid_norm_max_width()
 
 
@@ -796,3 +842,130 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pag
                                       heads_q, heads_kv, head_dim, scale, window, tile_rows=height)
     return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                            head_dim, scale, window)
+
+
+# --------------------------------------------------------------------------
+# a gated recurrence; latent attention
+# --------------------------------------------------------------------------
+def mingru_chunk_rows() -> int:
+    """Rows of a chunk of the recurrence's parallel form (the height of the runs of rows it takes)."""
+    return int(library.core().sb_mingru_chunk_rows())
+
+
+def mingru_scan(p: torch.Tensor, state: torch.Tensor, cu_rows: torch.Tensor, slots: torch.Tensor, n_seqs: int,
+                out_dtype: torch.dtype, chunks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """minGRU over a step's rows: ``p`` float32 [rows, 3 * width] holds the pre-activations of the
+    update gate, the candidate and the output gate; ``state`` float32 [slots, width] is read and
+    left moved on for the sequences ``slots`` [n_seqs] whose rows start at ``cu_rows``.  Returns
+    S_t * silu(g_t) [rows, width].  ``chunks`` (int32 [n, 4], runs of at most
+    :func:`mingru_chunk_rows` rows of one sequence in row order): the parallel form."""
+    _dev(p, state, cu_rows, slots, chunks)
+    if p.dtype != torch.float32 or p.dim() != 2 or p.shape[1] % 3:
+        raise KernelLibraryError("mingru_scan takes float32 rows [rows, 3 * width]")
+    rows, width = p.shape[0], p.shape[1] // 3
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != width:
+        raise KernelLibraryError(f"the recurrence's state must be float32 [slots, {width}]")
+    _i32(cu_rows, n_seqs + 1, "first rows of the sequences")
+    _i32(slots, n_seqs, "state rows of the sequences")
+    out = torch.empty((rows, width), dtype=out_dtype, device=p.device)
+    n_chunks, folded = 0, None
+    if chunks is not None:
+        if chunks.dtype != torch.int32 or chunks.dim() != 2 or chunks.shape[1] != 4:
+            raise KernelLibraryError("chunks must be int32 [n, 4]")
+        n_chunks = chunks.shape[0]
+        folded = torch.empty((n_chunks, width, 2), dtype=torch.float32, device=p.device)
+    check(library.core().sb_mingru_scan(_p(out), _dt(out), _p(p), _p(state), _p(cu_rows), _p(slots), n_seqs, rows,
+                                        width, _p(chunks), n_chunks, _p(folded), _stream()))
+    return out
+
+
+def latent_prepare(p: torch.Tensor, q_off: int, kv_off: int, act_dtype: torch.dtype, c_weight: Optional[torch.Tensor],
+                   eps: float, inv_freq: Optional[torch.Tensor], rot_dims: int, interleaved: bool,
+                   row_pos: torch.Tensor, row_seq: torch.Tensor, cache: Optional[torch.Tensor],
+                   page_table: Optional[torch.Tensor], heads: int, dim: int, rot_dim: int, rank: int):
+    """A step's rows of a latent-attention layer's input product ``p`` float32 [rows, n]: returns
+    (q_plain [rows, heads, dim], q_latent [rows, heads, rank + rot_dim] whose last rot_dim numbers
+    are the rotated query parts; the first rank are left for :func:`head_product`), and, with
+    ``kv_off`` >= 0, stores the normed latent and the rotated key part of every row at its
+    position in ``cache`` [pages, PAGE, rank + rot_dim]."""
+    _dev(p, c_weight, inv_freq, row_pos, row_seq, cache, page_table)
+    if p.dtype != torch.float32 or p.dim() != 2:
+        raise KernelLibraryError("latent_prepare takes float32 rows")
+    n, stride = p.shape
+    latent = rank + rot_dim
+    _i32(row_pos, n, "row positions")
+    _i32(row_seq, n, "row sequences")
+    if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() < rot_dims // 2):
+        raise KernelLibraryError("the rotation's table must be float32 with a number per pair")
+    max_pages = n_pages = 0
+    if kv_off >= 0:
+        if cache is None or page_table is None or cache.dim() != 3 or tuple(cache.shape[1:]) != (PAGE, latent):
+            raise KernelLibraryError(f"the latent cache must be [pages, {PAGE}, {latent}]")
+        if page_table.dtype != torch.int32 or page_table.dim() != 2:
+            raise KernelLibraryError("the page table must be int32 [sequences, pages]")
+        if c_weight is not None and c_weight.numel() != rank:
+            raise KernelLibraryError("the latent's norm weight does not match its size")
+        max_pages, n_pages = page_table.shape[1], cache.shape[0]
+    q_plain = torch.empty((n, heads, dim), dtype=act_dtype, device=p.device)
+    q_latent = torch.empty((n, heads, latent), dtype=act_dtype, device=p.device)
+    check(library.core().sb_latent_prepare(
+        _p(q_plain), _p(q_latent), _DT[act_dtype], _p(p), stride, int(q_off), int(kv_off), _p(c_weight),
+        _dt(c_weight) if c_weight is not None else 0, float(eps), _p(inv_freq), int(rot_dims), 1 if interleaved else 0,
+        _p(row_pos), _p(row_seq), _p(cache) if kv_off >= 0 else None, _dt(cache) if kv_off >= 0 else 0,
+        _p(page_table) if kv_off >= 0 else None, max_pages, n_pages, n, heads, dim, rot_dim, rank, _stream()))
+    return q_plain, q_latent
+
+
+def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, a, :n_out] = x[t, a, :] w[a] for every head a: ``x`` [rows, heads, n_in] (a view
+    whose last axis is dense), ``w`` [heads, n_in, n_out], ``out`` [rows, heads, >= n_out] (a view
+    likewise; only the first n_out numbers of a head are written); ``gate`` float32 [rows, >= heads *
+    n_out] (a view of rows): the result times sigmoid(gate)."""
+    for t in (x, w, out, gate):
+        if t is not None and not t.is_cuda:
+            raise KernelLibraryError("kernel operands must live on the GPU (there is no CPU path)")
+    if x.dim() != 3 or w.dim() != 3 or out.dim() != 3 or not w.is_contiguous():
+        raise KernelLibraryError("head_product takes x [rows, heads, in], w [heads, in, out], out [rows, heads, out]")
+    rows, heads, n_in = x.shape
+    n_out = w.shape[2]
+    if tuple(w.shape[:2]) != (heads, n_in) or out.shape[0] != rows or out.shape[1] != heads or out.shape[2] < n_out:
+        raise KernelLibraryError(f"head_product shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}, "
+                                 f"out {tuple(out.shape)}")
+    if x.stride(2) != 1 or out.stride(2) != 1 or x.dtype != w.dtype:
+        raise KernelLibraryError("head_product takes rows that are dense along their last axis, x and w of one type")
+    g_stride = 0
+    if gate is not None:
+        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != rows or gate.shape[1] < heads * n_out \
+                or gate.stride(1) != 1:
+            raise KernelLibraryError("the gate must be float32 [rows, heads * out]")
+        g_stride = gate.stride(0)
+    check(library.core().sb_head_product(_p(out), _dt(out), out.stride(0), out.stride(1), _p(x), _dt(x), x.stride(0),
+                                         x.stride(1), _p(w), _dt(w), _p(gate), g_stride, rows, heads, n_in, n_out,
+                                         _stream()))
+    return out
+
+
+def latent_attention_plain(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, row_pos: torch.Tensor,
+                           row_seq: torch.Tensor, rank: int, scale: float, window: int) -> torch.Tensor:
+    """Softmax attention of ``q`` [rows, heads, latent] over the cached rows [pages, PAGE, latent]
+    each row sees; returns the weighted sums of the rows' first ``rank`` numbers [rows, heads, rank]."""
+    _dev(q, cache, page_table, row_pos, row_seq)
+    if q.dim() != 3 or cache.dim() != 3 or cache.shape[1] != PAGE or cache.shape[2] != q.shape[2]:
+        raise KernelLibraryError("latent attention takes q [rows, heads, latent] and a cache [pages, PAGE, latent]")
+    n, heads, latent = q.shape
+    _i32(row_pos, n, "row positions")
+    _i32(row_seq, n, "row sequences")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("the page table must be int32 [sequences, pages]")
+    out = torch.empty((n, heads, rank), dtype=q.dtype, device=q.device)
+    check(library.core().sb_latent_attention(_p(out), _p(q), _dt(q), _p(cache), _dt(cache), _p(page_table),
+                                             page_table.shape[1], cache.shape[0], _p(row_pos), _p(row_seq), n, heads,
+                                             rank, latent - rank, float(scale), int(window), _stream()))
+    return out
+
+
+def latent_attention(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, ctx, rank: int, scale: float,
+                     window: int, fast: bool = True) -> torch.Tensor:
+    """Latent attention of a step's rows: the matrix-core kernels where they take the sizes and
+    types, else the kernel of one wave per (row, head)."""
+    return latent_attention_plain(q, cache, page_table, ctx.row_pos, ctx.row_seq, rank, scale, window)

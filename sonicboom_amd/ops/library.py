@@ -38,6 +38,16 @@ _CORE_SIGNATURES = {
     "sb_draw": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
     "sb_draw_after": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
     "sb_random_normal": [_P, _I, c_uint64, c_uint64, c_uint64, _I, c_double, c_double, _P],
+    "sb_rmsnorm_grouped": [_P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _P],
+    "sb_reduce_scaled_group_norm": [_P, _I, _P, _P, _I, _P, _I, _F, _P, _I, _I, _I, _I, _F, _I, _P],
+    "sb_add_scaled": [_P, _P, _I, _F, _Z, _P],
+    "sb_activate": [_P, _I, _P, _I, _Z, _I, _P, _I, _P],
+    "sb_mingru_chunk_rows": [],
+    "sb_mingru_scan": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _P, _I, _P, _P],
+    "sb_latent_prepare": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _F, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I,
+                          _I, _I, _I, _P],
+    "sb_head_product": [_P, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "sb_latent_attention": [_P, _P, _I, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {

@@ -2,4 +2,4 @@
 from .base import (CATEGORIES, KVSpec, Mixer, Part, RowsSpec, Runtime, StateSpec, build_part,  # noqa: F401
                    register_part, registered_parts)
 from .spec import ModelSpec, OrderEntry, PartSpec, TensorSpec  # noqa: F401
-from . import attention, block, embedding, ffn, norm, position  # noqa: F401
+from . import attention, block, embedding, ffn, latent_attention, norm, position, recurrent  # noqa: F401

@@ -8,7 +8,7 @@ multiplier (/root/reference/core/src/model/recipe.cpp:65-70, :165-167).
 Every size and switch is a parameter of the spec:
 
     heads_q, heads_kv, head_dim, window (0 = all keys), scale (None = 1/sqrt),
-    qkv_bias, out_bias
+    qkv_bias, out_bias, out_scale (the multiplier of the branch, 1 unless given)
 
 and the position encoding is a nested part.  The three input projections are
 packed into one matrix when the mixer is built, so a step runs one product
@@ -30,7 +30,7 @@ from .spec import PartSpec, TensorSpec
 
 def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_dim: int,
                    position: PartSpec, window: int = 0, scale: Optional[float] = None,
-                   qkv_bias: bool = True, out_bias: bool = False) -> PartSpec:
+                   qkv_bias: bool = True, out_bias: bool = False, out_scale: float = 1.0) -> PartSpec:
     qw, kvw = heads_q * head_dim, heads_kv * head_dim
     tensors = {
         "q_weight": TensorSpec(prefix + "q_proj.weight", (qw, width)),
@@ -47,6 +47,7 @@ def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_di
     return PartSpec("mixer", "attention", {
         "width": width, "heads_q": heads_q, "heads_kv": heads_kv, "head_dim": head_dim,
         "window": int(window), "scale": scale, "qkv_bias": qkv_bias, "out_bias": out_bias,
+        "out_scale": float(out_scale),
     }, tensors, {"position": position})
 
 
@@ -87,6 +88,7 @@ class Attention(Mixer):
         self._q_parts = (tensors["q_weight"], None if b_qkv is None else b_qkv[: self.q_width])
         self._q_only = None
         self.out = Linear(tensors["o_weight"], tensors.get("o_bias"), rt.fast_kernels)
+        self.out_scale = float(p.get("out_scale", 1.0))      # x += out_scale * attention(h)
 
     def query_only(self) -> None:
         """Build the queries-only projection (for run-order entries that read another entry's cache)."""
@@ -133,7 +135,7 @@ class Attention(Mixer):
             a = ops.attention_decode_rope(qkv, inv_freq, freq_factors, rot_dims, binding.k_cache, binding.v_cache,
                                           page_table, ctx.row_pos, self.heads_q, self.heads_kv, self.head_dim,
                                           self.scale, self.window, bias=bias, store=writes)
-            return self.out.add_into(a, x, then_norm, rt.act_dtype)
+            return self.out.add_into(a, x, then_norm, rt.act_dtype, scale=self.out_scale)
         q = ops.rope_kv_store(
             qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
             binding.k_cache if writes else None, binding.v_cache if writes else None,
@@ -141,4 +143,4 @@ class Attention(Mixer):
             bias=bias)
         a = ops.attention(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
                           self.head_dim, self.scale, self.window, fast=rt.fast_kernels, row_tile=self.row_tile)
-        return self.out.add_into(a, x, then_norm, rt.act_dtype)
+        return self.out.add_into(a, x, then_norm, rt.act_dtype, scale=self.out_scale)

@@ -3,7 +3,9 @@
 ``prenorm`` (/root/reference/core/src/model/emit.cpp:436-459 without the
 optional post-norms): x += mixer(norm(x)); x += ffn(norm(x)).  Mixer and
 feed-forward add their result into the float32 residual stream themselves,
-which lets their last projection fuse the addition.
+which lets their last projection fuse the addition (and a multiplier of the
+branch, the ``out_scale`` of their specs).  A block may have no feed-forward:
+it is then the first sublayer alone.
 """
 from __future__ import annotations
 
@@ -11,9 +13,13 @@ from .base import Part, register_part
 from .spec import PartSpec
 
 
-def prenorm_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec, ffn: PartSpec) -> PartSpec:
-    return PartSpec("block", "prenorm", {}, {}, {
-        "mixer_norm": mixer_norm, "mixer": mixer, "ffn_norm": ffn_norm, "ffn": ffn})
+def prenorm_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec = None, ffn: PartSpec = None) -> PartSpec:
+    parts = {"mixer_norm": mixer_norm, "mixer": mixer}
+    if ffn is not None:
+        if ffn_norm is None:
+            raise ValueError("a block with a feed-forward needs the norm before it")
+        parts.update(ffn_norm=ffn_norm, ffn=ffn)
+    return PartSpec("block", "prenorm", {}, {}, parts)
 
 
 @register_part("block", "prenorm")
@@ -25,8 +31,8 @@ class PreNormBlock(Part):
         self.mixer_norm = parts["mixer_norm"]
         self.first_norm = self.mixer_norm      # what the block before may apply in its last pass
         self.mixer = parts["mixer"]
-        self.ffn_norm = parts["ffn_norm"]
-        self.ffn = parts["ffn"]
+        self.ffn_norm = parts.get("ffn_norm")
+        self.ffn = parts.get("ffn")              # None: the block is its mixer's sublayer alone
 
     def forward(self, x, ctx, binding, h=None, next_norm=None):
         """Run the block on the residual stream ``x`` in place.  ``h`` is mixer_norm(x) when the
@@ -38,13 +44,16 @@ class PreNormBlock(Part):
         if h is None:
             h = self.mixer_norm.forward(x, act)
         f = None
+        after = self.ffn_norm if self.ffn is not None else next_norm     # the norm that follows the mixer
         if getattr(self.mixer, "fuses_norm", False):
-            f = self.mixer.forward(h, x, ctx, binding, then_norm=self.ffn_norm)
+            f = self.mixer.forward(h, x, ctx, binding, then_norm=after)
         else:
             self.mixer.forward(h, x, ctx, binding)
         trace = getattr(ctx, "trace", None)
         if trace is not None:
             trace("after_mixer", x)
+        if self.ffn is None:
+            return f
         if f is None:
             f = self.ffn_norm.forward(x, act)
         out = None

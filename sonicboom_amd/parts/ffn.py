@@ -1,4 +1,6 @@
-"""Gated dense feed-forward: y = W_down (act(W_gate f) * (W_up f)).
+"""Dense feed-forwards, gated and plain.
+
+``gated_dense``: y = W_down (act(W_gate f) * (W_up f)).
 
 /root/reference/core/src/model/emit.cpp:364-374; the activation is a parameter
 of the spec: "silu", g / (1 + exp(-g)) (/root/reference/core/src/nn/activation.cpp:41-50),
@@ -7,11 +9,19 @@ kernels apply either in their epilogue.  The gate and up matrices
 are stacked into one [2*inner, width] matrix when the part is built, so a
 step runs one product for both; its float32 result feeds the activation
 kernel, whose output is rounded once to the activation type.
+
+``dense``: y = W_down act(W_up f), the activation one of ``ops.ACTIVATIONS``; "xielu" reads its two
+numbers (p, q) from a tensor of the layer: softplus(p) z^2 + z/2 for z > 0 and
+(1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 else.  The up product leaves in float32, the activation
+kernel rounds once to the activation type.
+
+Both add ``out_scale`` times their result into the stream (1 unless the spec says otherwise).
 """
 from __future__ import annotations
 
 import torch
 
+from .. import ops
 from .base import Part, register_part
 from .linear import Linear
 from .spec import PartSpec, TensorSpec
@@ -19,8 +29,9 @@ from .spec import PartSpec, TensorSpec
 ACTIVATIONS = ("silu", "gelu_tanh")    # the gates the product kernels apply in their epilogue
 
 
-def gated_ffn_spec(prefix: str, width: int, inner: int, activation: str = "silu") -> PartSpec:
-    return PartSpec("ffn", "gated_dense", {"width": width, "inner": inner, "activation": activation}, {
+def gated_ffn_spec(prefix: str, width: int, inner: int, activation: str = "silu", out_scale: float = 1.0) -> PartSpec:
+    return PartSpec("ffn", "gated_dense", {"width": width, "inner": inner, "activation": activation,
+                                           "out_scale": float(out_scale)}, {
         "gate_weight": TensorSpec(prefix + "gate_proj.weight", (inner, width)),
         "up_weight": TensorSpec(prefix + "up_proj.weight", (inner, width)),
         "down_weight": TensorSpec(prefix + "down_proj.weight", (width, inner)),
@@ -44,12 +55,51 @@ class GatedDenseFFN(Part):
         self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=True,
                               activation=self.activation)
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
+        self.out_scale = float(p.get("out_scale", 1.0))
 
     fuses_norm = True
     graph_safe = True     # its launches depend on device buffers only
 
     def forward(self, h, x, ctx, then_norm=None):
-        """x += ffn(h).  Returns then_norm(x) when the down projection could apply the norm in
-        its last pass, else None."""
+        """x += out_scale * ffn(h).  Returns then_norm(x) when the down projection could apply the
+        norm in its last pass, else None."""
         mid = self.gate_up.gated_product(h, self.rt.act_dtype)
-        return self.down.add_into(mid, x, then_norm, self.rt.act_dtype)
+        return self.down.add_into(mid, x, then_norm, self.rt.act_dtype, scale=self.out_scale)
+
+
+def dense_ffn_spec(up_name: str, down_name: str, width: int, inner: int, activation: str,
+                   act_name: str = None, out_scale: float = 1.0) -> PartSpec:
+    """``act_name``: the tensor that holds the activation's numbers (xIELU's two)."""
+    tensors = {"up_weight": TensorSpec(up_name, (inner, width)), "down_weight": TensorSpec(down_name, (width, inner))}
+    if act_name is not None:
+        tensors["act_params"] = TensorSpec(act_name, (2,), init=(0.0, 0.5))
+    return PartSpec("ffn", "dense", {"width": width, "inner": inner, "activation": activation,
+                                     "out_scale": float(out_scale)}, tensors)
+
+
+@register_part("ffn", "dense")
+class DenseFFN(Part):
+    category = "ffn"
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        p = spec.params
+        self.width, self.inner = int(p["width"]), int(p["inner"])
+        self.activation = p["activation"]
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {self.activation!r}; known: {sorted(ops.ACTIVATIONS)}")
+        self.act_params = tensors.get("act_params")
+        if self.activation == "xielu" and self.act_params is None:
+            raise ValueError("xIELU needs the tensor with its two numbers")
+        self.up = Linear(tensors["up_weight"], None, rt.fast_kernels)
+        self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
+        self.out_scale = float(p.get("out_scale", 1.0))
+
+    fuses_norm = True
+    graph_safe = True     # its launches depend on device buffers only
+
+    def forward(self, h, x, ctx, then_norm=None):
+        """x += out_scale * W_down act(W_up h).  Returns then_norm(x) when the down projection could
+        apply the norm in its last pass, else None."""
+        mid = ops.activate(self.up(h, torch.float32), self.rt.act_dtype, self.activation, self.act_params)
+        return self.down.add_into(mid, x, then_norm, self.rt.act_dtype, scale=self.out_scale)

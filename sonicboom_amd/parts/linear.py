@@ -72,15 +72,21 @@ class Linear:
             return None
         return ops.gemm_bf16_partial(x, self.packed, packed_shape=(self.rows, self.n_in))
 
-    def add_into(self, x: torch.Tensor, resid: torch.Tensor, then_norm=None, out_dtype=None):
-        """resid += x W^T (+ b).  With ``then_norm`` (an RMS norm part) tries to return
-        then_norm(resid) in ``out_dtype`` from the same pass; None when the caller has to norm."""
+    def add_into(self, x: torch.Tensor, resid: torch.Tensor, then_norm=None, out_dtype=None, scale: float = 1.0):
+        """resid += scale * (x W^T (+ b)).  With ``then_norm`` (an RMS norm part, whole rows or in
+        groups) tries to return then_norm(resid) in ``out_dtype`` from the same pass; None when the
+        caller has to norm."""
         part = self.partial(x)
-        if part is not None and ops.reduce_resid_norm_ok(self.n_out):
-            fuse = then_norm is not None and getattr(then_norm, "fusable", False)
+        fuse = then_norm is not None and getattr(then_norm, "fusable", False)
+        groups = int(getattr(then_norm, "groups", 1)) if fuse else 1
+        if part is not None and ops.reduce_resid_norm_ok(self.n_out, scale, groups):
             return ops.reduce_resid_norm(part, self.bias, resid, then_norm.weight if fuse else None,
-                                         then_norm.eps if fuse else 0.0, out_dtype if fuse else None)
-        self(x, torch.float32, resid=resid, out=resid)
+                                         then_norm.eps if fuse else 0.0, out_dtype if fuse else None,
+                                         scale=scale, groups=groups)
+        if scale == 1.0:
+            self(x, torch.float32, resid=resid, out=resid)
+        else:
+            ops.add_scaled(resid, self(x, torch.float32), scale)
         return None
 
     def gated_product(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

@@ -7,6 +7,10 @@ attention scale — are parameters; the per-pair factor
 ``expf(-2 i / n * logf(base))`` is computed here in float32 exactly as the
 reference writes it and handed to the kernel as a table.
 
+``rope_interleaved``: the same rotation on neighbouring pairs (2i, 2i + 1) of the first
+``rot_dims`` numbers, pair i turning by position * base^(-2i / rot_dims); for mixers whose
+kernels take the pairing as an argument.
+
 ``none``: no encoding.
 """
 from __future__ import annotations
@@ -65,9 +69,14 @@ def scaled_rope_tables(kind: str, factor: float, head_dim: int, base: float, ori
     return table, score
 
 
+def rope_interleaved_spec(rot_dims: int, base: float) -> PartSpec:
+    return PartSpec("position", "rope_interleaved", {"rot_dims": int(rot_dims), "base": float(base)})
+
+
 class Position(Part):
     category = "position"
     score_scale = 1.0
+    interleaved = False     # rotary encodings: pairs are (i, i + rot_dims / 2); True: (2i, 2i + 1)
 
     def rotary_tables(self):
         """(inv_freq, freq_factors, rot_dims) for the fused rotate-and-store
@@ -113,3 +122,23 @@ class Rope(Position):
 
     def rotary_tables(self):
         return (self.inv_freq, self.freq_factors, self.rot_dims)
+
+
+@register_part("position", "rope_interleaved")
+class RopeInterleaved(Position):
+    """Pairs (2i, 2i + 1), i < rot_dims / 2, turn by position * f_i, f_i = base^(-2i / rot_dims)
+    computed in float64 and rounded once to the float32 table the kernels multiply positions with."""
+    interleaved = True
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        self.rot_dims = int(spec.params["rot_dims"])
+        if self.rot_dims < 0 or self.rot_dims % 2:
+            raise ValueError(f"rotary width {self.rot_dims} must be even")
+        base = float(spec.params["base"])
+        i = np.arange(self.rot_dims // 2, dtype=np.float64)
+        inv = np.power(np.float64(base), -2.0 * i / max(self.rot_dims, 1)).astype(np.float32)
+        self.inv_freq = torch.from_numpy(inv).to(rt.device) if self.rot_dims else None
+
+    def rotary_tables(self):
+        return (self.inv_freq, None, self.rot_dims)
