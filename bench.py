@@ -28,6 +28,14 @@ loop itself: ``--sizes 14b``: 16 prompts of seeded lengths uniform in [256, 4096
 8192 tokens a sequence, prompts in one step, then 256 greedy steps; ``--sizes 72b``: 8 prompts of
 512 to 2048 tokens, 128 steps, 4096 tokens a sequence.  Prefill and decode are timed apart.
 
+``--workload designs`` runs the Rasizen design (gated recurrences and latent attention) at a few
+layer sizes that resemble a real model's (``--design-sizes``: widths) beside the Qwen2.5 design at
+the same width, head count and feed-forward weight count: prefill of one ``--prompt``-token prompt
+and decode of ``--batch`` sequences at that depth, tokens a second, and the time of every kernel of
+one prompt step and one decode step with what it reaches of its roofline (bytes it must move over
+8 TB/s, or flops over the dense bf16 peak, whichever is the larger time).  A table goes to standard
+error, one JSON line to standard output.
+
 ``--workload forms`` prints a table instead of the line: the decode step (``--batches 1,8``) with
 the qkv, output and down product forced, one at a time, to every form (waves a block x K slices)
 of the kernel that streams the weights, against the launchers' own choices.
@@ -249,7 +257,9 @@ def main() -> int:
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b", help="layer sizes (default: the benchmark's)")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
-    ap.add_argument("--workload", choices=("steady", "mixed", "forms"), default="steady")
+    ap.add_argument("--workload", choices=("steady", "mixed", "forms", "designs"), default="steady")
+    ap.add_argument("--design-sizes", default="2048,4096",
+                    help="--workload designs: the widths of the layer sizes to run, comma separated")
     ap.add_argument("--batches", default="1,8", help="--workload forms: the batch sizes, comma separated")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel")
@@ -275,6 +285,9 @@ def main() -> int:
             elif not arg.startswith("--runs="):
                 argv.append(arg)
         return median_of_runs(argv, a.runs)
+
+    if a.workload == "designs":
+        return design_comparison(a)
 
     import numpy as np
     import torch
@@ -622,6 +635,209 @@ def main() -> int:
         line["prefix_reuse"] = prefix_reuse
     result_lines(line)
     print(json.dumps(line), flush=True)
+    return 0
+
+
+# ---- the designs side by side --------------------------------------------------------------------
+def rasizen_sizes(width, n_blocks=2, window=4096, vocab=32768):
+    """Layer sizes in the manner of a real model of this width: heads of 128 plain + 64 rotated
+    numbers and 128 values, a latent of 512, an ungated feed-forward of 4 widths, recurrences of 2
+    widths; a block of four layers = recurrence, attention with its own latent, attention that
+    reads it, recurrence; the attention layers carry the feed-forwards."""
+    heads = width // 128
+    att = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+           "mask": {"size": window}, "rot": {"base": 1e6, "dims": 64}}
+    layers = []
+    for b in range(n_blocks):
+        own = len(layers) + 1
+        layers += [{"type": "mingru", "mixer": {"width": 2 * width}, "mlp": None},
+                   {"type": "latent_attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": 4 * width}},
+                   {"type": "latent_attention", "mixer": dict(att, kv_from=own), "mlp": {"kind": "dense", "ff": 4 * width}},
+                   {"type": "mingru", "mixer": {"width": 2 * width}, "mlp": None}]
+    return {"architecture": "Rasizen", "vocab": vocab, "width": width, "residual_mult": 0.5,
+            "norm": {"eps": 1e-5, "groups": 2}, "layers": layers}
+
+
+def qwen_sizes(width, n_layers=4, vocab=32768):
+    """The Qwen2.5 design at the same width and head count, a gated feed-forward of the same weight
+    count as the ungated one of 4 widths (inner 8/3 widths, in 256s), a quarter of the heads as kv heads."""
+    heads = width // 128
+    return dict(CONFIG_7B, num_hidden_layers=n_layers, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), intermediate_size=(8 * width // 3 + 255) // 256 * 256,
+                vocab_size=vocab, tie_word_embeddings=True)
+
+
+class AllOpsTimer:
+    """Times every launching function of ``sonicboom_amd.ops`` between two events, summed by
+    (function, what tells its calls apart: a product's matrix, the rows)."""
+
+    SKIP = ("pack_weight", "read_bandwidth", "random_normal", "attention_row_tile", "attention_row_tiles",
+            "attention_tall_ok", "attention_mfma_ok", "attention_decode_rope_ok", "gate_code", "reduce_resid_norm_ok",
+            "attention_decode_pages_per_wave", "gemm_tile_shape", "gemm_few_rows_kernel", "mingru_chunk_rows",
+            "loaded_paths", "check", "latent_attention_mfma_ok")
+    INNER = ("attention_plain", "attention_decode_mfma", "attention_prefill_mfma", "latent_attention_plain",
+             "latent_attention_mfma")      # called by the dispatchers that are timed themselves
+
+    def __init__(self):
+        self.records, self._saved = [], {}
+
+    def __enter__(self):
+        import inspect
+
+        import torch
+        from sonicboom_amd import ops
+        from sonicboom_amd.ops import kernels
+        for name, fn in vars(kernels).items():
+            if name.startswith("_") or name in self.SKIP or name in self.INNER or not inspect.isfunction(fn) \
+                    or fn.__module__ != kernels.__name__:
+                continue
+            self._saved[name] = fn
+
+            def timed(*args, _fn=fn, _name=name, **kw):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = _fn(*args, **kw)
+                e1.record()
+                if out is not None or not _name.startswith("gemm_bf16"):
+                    label = _name
+                    if _name.startswith("gemm"):
+                        n, k = kw.get("packed_shape") or (args[1].shape[0], args[1].shape[-1])
+                        label = f"{_name} {n}x{k}"
+                    elif _name == "head_product":
+                        label = f"{_name} {tuple(args[1].shape)}"
+                    self.records.append((label, e0, e1))
+                return out
+            setattr(ops, name, timed)
+            setattr(kernels, name, timed)
+        return self
+
+    def __exit__(self, *exc):
+        from sonicboom_amd import ops
+        from sonicboom_amd.ops import kernels
+        for name, fn in self._saved.items():
+            setattr(ops, name, fn)
+            setattr(kernels, name, fn)
+
+    def totals(self):
+        import torch
+        torch.cuda.synchronize()
+        out = {}
+        for label, e0, e1 in self.records:
+            us, n = out.get(label, (0.0, 0))
+            out[label] = (us + e0.elapsed_time(e1) * 1e3, n + 1)
+        return out
+
+
+def design_roofline(label, us, calls, rows, depth, batch, width, cfgs):
+    """(share of the roofline reached, what bounds it) for the kernels whose work is easy to count:
+    per call, the bytes it must move over 8 TB/s against the flops over the dense bf16 peak."""
+    per = us / calls * 1e-6
+    peak_b, peak_f = PEAK_HBM_GBS * 1e9, PEAK_FLOPS["bf16"]
+    decode = rows == batch
+    keys = min(depth, cfgs["window"])
+    H, rank, rot = cfgs["heads"], cfgs["rank"], cfgs["rot"]
+    nbytes = flops = None
+    if label.startswith("gemm"):
+        n, k = (int(v) for v in label.split()[-1].split("x"))
+        nbytes, flops = 2 * n * k + 2 * rows * k + 4 * rows * (n // (2 if "gated" in label else 1)), 2 * rows * n * k
+    elif label.startswith("rmsnorm") or label == "reduce_resid_norm":
+        nbytes = rows * width * (4 + 2 + (8 if label == "reduce_resid_norm" else 0))
+    elif label == "mingru_scan":
+        nbytes = rows * cfgs["gru"] * (12 + 2)
+    elif label == "activate":
+        nbytes = rows * cfgs["ff"] * (4 + 2)
+    elif label == "latent_prepare":
+        nbytes = rows * (4 * (H * 192 + rank + rot) + 2 * (H * (192 + rank) + rank + rot))
+    elif label.startswith("head_product"):
+        a, i, o = (int(v) for v in label.split("(")[1].rstrip(")").split(","))
+        nbytes, flops = 2 * a * i * o + 2 * rows * a * (i + o), 2 * rows * a * i * o
+    elif label == "latent_attention":
+        pairs = batch * keys if decode else sum(min(t + 1, cfgs["window"]) for t in range(rows))
+        flops = 2 * pairs * H * (2 * rank + rot)
+        nbytes = (batch * keys if decode else rows) * 2 * (rank + rot) + 2 * rows * H * (2 * rank + rot)
+    elif label in ("attention", "attention_decode_rope"):
+        pairs = batch * depth if decode else rows * (rows + 1) // 2
+        flops = 4 * pairs * H * 128
+        nbytes = (batch * depth if decode else rows) * 2 * 2 * cfgs["kvw"] + 4 * rows * H * 128
+    elif label == "rope_kv_store":
+        nbytes = rows * (H * 128 + 2 * cfgs["kvw"]) * (4 + 2)
+    if nbytes is None and flops is None:
+        return None, ""
+    tb, tf = (nbytes or 0) / peak_b, (flops or 0) / peak_f
+    return max(tb, tf) / per, "bytes" if tb >= tf else "flops"
+
+
+def design_comparison(a) -> int:
+    import numpy as np
+    import torch
+
+    from sonicboom_amd.engine import DecoderModel, Engine, StepEntry
+
+    rng = np.random.default_rng(0)
+    out, table = {}, []
+    for width in (int(v) for v in a.design_sizes.split(",")):
+        for design, cfg in (("rasizen", rasizen_sizes(width)), ("qwen2", qwen_sizes(width))):
+            model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
+            heads = width // 128
+            cfgs = {"heads": heads, "rank": 512, "rot": 64, "window": 4096 if design == "rasizen" else 1 << 30,
+                    "gru": 2 * width, "ff": 4 * width, "kvw": max(1, heads // 4) * 128}
+            eng = Engine(model, (a.prompt + a.steps + a.warmup + 128) * (a.batch + 1), max_positions=0)
+            prompt = [int(t) for t in rng.integers(0, cfg.get("vocab", cfg.get("vocab_size")), size=a.prompt)]
+
+            def prefill_once(timer=None):
+                slot = eng.alloc_slot()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                eng.step([StepEntry(slot, prompt, [a.prompt - 1])])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t0
+                eng.free_slot(slot)
+                return dt
+            for _ in range(2):
+                prefill_once()
+            prefill_s = statistics.median(prefill_once() for _ in range(5))
+            with AllOpsTimer() as tm:
+                prefill_once()
+                pre_kernels = tm.totals()
+            # decode: a batch at the prompt's depth, through the recorded step
+            slots = [eng.alloc_slot() for _ in range(a.batch)]
+            eng.step([StepEntry(s, prompt, ()) for s in slots])
+            loop = eng.decode_loop()
+            loop.start(slots, [1] * a.batch)
+            for _ in range(a.warmup):
+                loop.step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(a.steps):
+                loop.step()
+            torch.cuda.synchronize()
+            step_s = (time.perf_counter() - t0) / a.steps
+            with AllOpsTimer() as tm:
+                eng.step([StepEntry(s, [1], [0]) for s in slots])
+                dec_kernels = tm.totals()
+            for s in slots:
+                eng.free_slot(s)
+            key = f"{design}_{width}"
+            out[key] = {"prefill_tokens_per_s": round(a.prompt / prefill_s, 1), "decode_tokens_per_s": round(a.batch / step_s, 1),
+                        "prefill_ms": round(prefill_s * 1e3, 3), "decode_step_ms": round(step_s * 1e3, 3),
+                        "layers": len(model.order), "kernels": {}}
+            for phase, totals, rows in (("prefill", pre_kernels, a.prompt), ("decode", dec_kernels, a.batch)):
+                for label, (us, calls) in sorted(totals.items(), key=lambda kv: -kv[1][0]):
+                    share, bound = design_roofline(label.replace("gemm_bf16_partial", "gemm").replace("gemm_bf16", "gemm"),
+                                                   us, calls, rows, a.prompt, a.batch, width, cfgs)
+                    out[key]["kernels"][f"{phase}: {label}"] = {"us": round(us, 1), "calls": calls,
+                                                                "of_roofline": None if share is None else round(share, 3)}
+                    table.append(f"| {key} | {phase} | {label} | {calls} | {us / calls:.1f} | "
+                                 f"{'' if share is None else f'{share:.3f} ({bound})'} |")
+            del eng, model, loop
+            torch.cuda.empty_cache()
+    print("| model | step | kernel | calls | us a call | of its roofline |\n|---|---|---|---|---|---|", file=sys.stderr)
+    print("\n".join(table), file=sys.stderr)
+    for key, v in out.items():
+        print(f"RESULT {key} prefill_tokens_per_s={v['prefill_tokens_per_s']} decode_tokens_per_s={v['decode_tokens_per_s']} "
+              f"prefill_ms={v['prefill_ms']} decode_step_ms={v['decode_step_ms']}", file=sys.stderr)
+    print(json.dumps({"workload": "designs", "prompt": a.prompt, "batch": a.batch, "steps": a.steps, "dtype": "bf16",
+                      "data": "synthetic", "models": out}))
     return 0
 
 

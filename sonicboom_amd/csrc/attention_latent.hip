@@ -13,7 +13,7 @@
 //
 //   sb_latent_prepare    a step's rows of the input product: norm and store c, rotate and store r,
 //                        rotate the queries' rotated parts, split off their plain parts
-//   sb_head_product      out[t, a, :] = in[t, a, :] W[a], one small matrix per head
+//   sb_head_product      out[t, a, :] = W[a] in[t, a, :], one small matrix per head
 //   sb_latent_attention  one wave per (row, head), 64 keys at a time, softmax in float32 whose
 //                        order of sums depends on key positions only: the 32-bit path, and the
 //                        bfloat16 path for sizes the matrix-core kernel does not take
@@ -109,7 +109,7 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
   }
 }
 
-// out[t, a, o] = sum_i in[t, a, i] W[a][i][o]  (times sigmoid(gate[t, a * n_out + o]) when gated).
+// out[t, a, o] = sum_i W[a][o][i] in[t, a, i]  (times sigmoid(gate[t, a * n_out + o]) when gated).
 // A block takes kHeadRows rows of one head; the rows' inputs wait in LDS, a thread owns output
 // columns and sums in ascending i from zero, so an element's bits do not depend on the batch.
 constexpr int kHeadRows = 8;
@@ -134,8 +134,9 @@ head_product_kernel(TO *__restrict__ out, int out_stride, int out_hstride, const
     float acc[kHeadRows];
 #pragma unroll
     for (int r = 0; r < kHeadRows; ++r) acc[r] = 0.0f;
+    const TW *wr = wa + size_t(o) * n_in;
     for (int i = 0; i < n_in; ++i) {
-      const float wv = ld_f(wa, size_t(i) * n_out + o);
+      const float wv = ld_f(wr, i);
 #pragma unroll
       for (int r = 0; r < kHeadRows; ++r) acc[r] = fmaf(xin[r * n_in + i], wv, acc[r]);
     }
@@ -264,7 +265,7 @@ extern "C" int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, c
   return sb::check_launch("sb_latent_prepare");
 }
 
-// out[t, a, o] = sum_i in[t, a, i] W[a][i][o] for heads a, W [heads, n_in, n_out] (input-major);
+// out[t, a, o] = sum_i W[a][o][i] in[t, a, i] for heads a, W [heads, n_out, n_in];
 // element (t, a, .) of out lies at t * out_stride + a * out_hstride, of in at t * in_stride +
 // a * in_hstride.  gate (f32, or NULL): the result is multiplied by sigmoid(gate[t * gate_stride +
 // a * n_out + o]).  in and W of one type (f32 or bf16), out f32 or bf16.

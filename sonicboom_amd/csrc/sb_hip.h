@@ -198,7 +198,7 @@ int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, const float 
                       const int32_t *row_seq, void *cache, int cache_dtype, const int32_t *page_table,
                       int max_pages, int n_pages_total, int n_rows, int heads, int dim, int rot_dim,
                       int rank, void *stream);
-/* out[t, a, o] = sum_i in[t, a, i] W[a][i][o], W [heads, n_in, n_out]; (t, a, .) of out at
+/* out[t, a, o] = sum_i W[a][o][i] in[t, a, i], W [heads, n_out, n_in]; (t, a, .) of out at
  * t * out_stride + a * out_hstride, of in at t * in_stride + a * in_hstride; gate f32 or NULL:
  * times sigmoid(gate[t * gate_stride + a * n_out + o]). */
 int sb_head_product(void *out, int out_dtype, int out_stride, int out_hstride, const void *in,
@@ -212,6 +212,21 @@ int sb_latent_attention(void *out, const void *q, int act_dtype, const void *cac
                         const int32_t *page_table, int max_pages, int n_pages_total,
                         const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads, int rank,
                         int rot_dim, float scale, int window, void *stream);
+
+/* The same two on the matrix cores, everything bfloat16 (csrc/attention_latent_mfma.hip); the
+ * *_ok functions say whether the sizes are taken.  tiles int32 [n_tiles, 4] = (first row, rows,
+ * sequence, 0): runs of up to tile_rows consecutive rows of a sequence, tile_rows 16 (a wave takes 16
+ * rows of a head) or 1 (16 heads of a row). */
+int sb_head_product_bf16_ok(int out_stride, int out_hstride, int in_stride, int in_hstride, int n_in);
+int sb_head_product_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride,
+                         int in_hstride, const void *w, const float *gate, int gate_stride, int n_rows,
+                         int heads, int n_in, int n_out, void *stream);
+int sb_latent_attention_tile_rows(void);
+int sb_latent_attention_bf16_ok(int rank, int rot_dim);
+int sb_latent_attention_bf16(void *out, const void *q, const void *cache, const int32_t *page_table,
+                             int max_pages, int n_pages_total, const int32_t *row_pos, const int32_t *tiles,
+                             int n_tiles, int heads, int rank, int rot_dim, float scale, int window,
+                             int tile_rows, void *stream);
 
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts

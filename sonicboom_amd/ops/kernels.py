@@ -916,19 +916,21 @@ def latent_prepare(p: torch.Tensor, q_off: int, kv_off: int, act_dtype: torch.dt
     return q_plain, q_latent
 
 
-def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, a, :n_out] = x[t, a, :] w[a] for every head a: ``x`` [rows, heads, n_in] (a view
-    whose last axis is dense), ``w`` [heads, n_in, n_out], ``out`` [rows, heads, >= n_out] (a view
+def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None,
+                 fast: bool = True) -> torch.Tensor:
+    """out[t, a, :n_out] = w[a] x[t, a, :] for every head a: ``x`` [rows, heads, n_in] (a view
+    whose last axis is dense), ``w`` [heads, n_out, n_in], ``out`` [rows, heads, >= n_out] (a view
     likewise; only the first n_out numbers of a head are written); ``gate`` float32 [rows, >= heads *
-    n_out] (a view of rows): the result times sigmoid(gate)."""
+    n_out] (a view of rows): the result times sigmoid(gate).  bfloat16 operands whose inner size and
+    strides are multiples of 8 run on the matrix cores (``fast``), the rest on the plain kernel."""
     for t in (x, w, out, gate):
         if t is not None and not t.is_cuda:
             raise KernelLibraryError("kernel operands must live on the GPU (there is no CPU path)")
     if x.dim() != 3 or w.dim() != 3 or out.dim() != 3 or not w.is_contiguous():
-        raise KernelLibraryError("head_product takes x [rows, heads, in], w [heads, in, out], out [rows, heads, out]")
+        raise KernelLibraryError("head_product takes x [rows, heads, in], w [heads, out, in], out [rows, heads, out]")
     rows, heads, n_in = x.shape
-    n_out = w.shape[2]
-    if tuple(w.shape[:2]) != (heads, n_in) or out.shape[0] != rows or out.shape[1] != heads or out.shape[2] < n_out:
+    n_out = w.shape[1]
+    if w.shape[0] != heads or w.shape[2] != n_in or out.shape[0] != rows or out.shape[1] != heads or out.shape[2] < n_out:
         raise KernelLibraryError(f"head_product shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}, "
                                  f"out {tuple(out.shape)}")
     if x.stride(2) != 1 or out.stride(2) != 1 or x.dtype != w.dtype:
@@ -939,9 +941,15 @@ def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Opti
                 or gate.stride(1) != 1:
             raise KernelLibraryError("the gate must be float32 [rows, heads * out]")
         g_stride = gate.stride(0)
-    check(library.core().sb_head_product(_p(out), _dt(out), out.stride(0), out.stride(1), _p(x), _dt(x), x.stride(0),
-                                         x.stride(1), _p(w), _dt(w), _p(gate), g_stride, rows, heads, n_in, n_out,
-                                         _stream()))
+    lib = library.core()
+    if fast and x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 \
+            and w.data_ptr() % 16 == 0 and lib.sb_head_product_bf16_ok(out.stride(0), out.stride(1), x.stride(0),
+                                                                       x.stride(1), n_in):
+        check(lib.sb_head_product_bf16(_p(out), out.stride(0), out.stride(1), _p(x), x.stride(0), x.stride(1), _p(w),
+                                       _p(gate), g_stride, rows, heads, n_in, n_out, _stream()))
+        return out
+    check(lib.sb_head_product(_p(out), _dt(out), out.stride(0), out.stride(1), _p(x), _dt(x), x.stride(0),
+                              x.stride(1), _p(w), _dt(w), _p(gate), g_stride, rows, heads, n_in, n_out, _stream()))
     return out
 
 
@@ -964,8 +972,41 @@ def latent_attention_plain(q: torch.Tensor, cache: torch.Tensor, page_table: tor
     return out
 
 
+LATENT_ROW_TILE = 16        # rows of a run that a prompt step's matrix-core launch takes (sb_latent_attention_tile_rows)
+
+
+def latent_attention_mfma_ok(q_dtype, cache_dtype, rank: int, rot_dim: int) -> bool:
+    return q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 \
+        and bool(library.core().sb_latent_attention_bf16_ok(int(rank), int(rot_dim)))
+
+
+def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, row_pos: torch.Tensor,
+                          tiles: torch.Tensor, rank: int, scale: float, window: int, single_rows: bool) -> torch.Tensor:
+    """The matrix-core form: ``tiles`` int32 [n, 4], runs of up to 16 consecutive rows of a sequence;
+    ``single_rows``: every run is one row (a decode step), a wave then takes 16 heads of it."""
+    _dev(q, cache, page_table, row_pos, tiles)
+    n, heads, latent = q.shape
+    if cache.dim() != 3 or cache.shape[1] != PAGE or cache.shape[2] != latent:
+        raise KernelLibraryError("latent attention takes q [rows, heads, latent] and a cache [pages, PAGE, latent]")
+    _i32(row_pos, n, "row positions")
+    if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 4:
+        raise KernelLibraryError("row tiles must be int32 [n, 4]")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("the page table must be int32 [sequences, pages]")
+    out = torch.empty((n, heads, rank), dtype=q.dtype, device=q.device)
+    check(library.core().sb_latent_attention_bf16(_p(out), _p(q), _p(cache), _p(page_table), page_table.shape[1],
+                                                  cache.shape[0], _p(row_pos), _p(tiles), tiles.shape[0], heads, rank,
+                                                  latent - rank, float(scale), int(window), 1 if single_rows else 16,
+                                                  _stream()))
+    return out
+
+
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, ctx, rank: int, scale: float,
                      window: int, fast: bool = True) -> torch.Tensor:
-    """Latent attention of a step's rows: the matrix-core kernels where they take the sizes and
-    types, else the kernel of one wave per (row, head)."""
+    """Latent attention of a step's rows: the matrix-core kernel where it takes the sizes and
+    types (the step's context then lists the rows in runs of LATENT_ROW_TILE), else the kernel of
+    one wave per (row, head)."""
+    if fast and latent_attention_mfma_ok(q.dtype, cache.dtype, rank, q.shape[2] - rank):
+        return latent_attention_mfma(q, cache, page_table, ctx.row_pos, ctx.row_tiles(LATENT_ROW_TILE), rank, scale,
+                                     window, single_rows=bool(ctx.is_decode))
     return latent_attention_plain(q, cache, page_table, ctx.row_pos, ctx.row_seq, rank, scale, window)

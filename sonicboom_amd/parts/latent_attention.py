@@ -83,11 +83,14 @@ class LatentAttention(Mixer):
         self.kv_off = self.g_off + H * self.vdim if self.own_latent else -1
         self.proj = Linear(torch.cat(ws, dim=0), None, rt.fast_kernels)
         self.c_weight = tensors.get("dkv_norm")
-        # per head a small matrix, input-major: W_uk,a [dim, rank] as the file has it (keys = W_uk c, so
-        # W_uk,a^T carries a query into the latent space); W_uv,a turned to [rank, vdim]
+        # per head a small matrix [out, in]: keys are W_uk c, so W_uk,a^T [rank, dim] carries head a's plain
+        # query part into the latent space; W_uv,a [vdim, rank] as the file has it brings a result back
         wdt = rt.act_dtype
-        self.uk = tensors["uk_weight"].to(wdt).reshape(H, self.dim, self.rank).contiguous()
-        self.uv = tensors["uv_weight"].to(wdt).reshape(H, self.vdim, self.rank).transpose(1, 2).contiguous()
+        self.uk = tensors["uk_weight"].to(wdt).reshape(H, self.dim, self.rank).transpose(1, 2).contiguous()
+        self.uv = tensors["uv_weight"].to(wdt).reshape(H, self.vdim, self.rank).contiguous()
+        # the matrix-core attention kernel takes a prompt step's rows in runs of this many
+        if rt.fast_kernels and ops.latent_attention_mfma_ok(rt.act_dtype, rt.cache_dtype, self.rank, self.rot_dim):
+            self.row_tile = ops.LATENT_ROW_TILE
         self.out = Linear(tensors["o_weight"], None, rt.fast_kernels)
 
     def cache_spec(self) -> RowsSpec:
@@ -107,9 +110,9 @@ class LatentAttention(Mixer):
             pre, self.q_off, self.kv_off, rt.act_dtype, self.c_weight, self.eps, self.inv_freq, self.rot_dims,
             bool(self.position.interleaved), ctx.row_pos, ctx.row_seq, cache if writes else None,
             table if writes else None, self.heads, self.dim, self.rot_dim, self.rank)
-        ops.head_product(q_plain, self.uk, q_lat)          # the first rank numbers of every head's query
+        ops.head_product(q_plain, self.uk, q_lat, fast=rt.fast_kernels)     # the first rank numbers of every head's query
         a_lat = ops.latent_attention(q_lat, cache, table, ctx, self.rank, self.scale, self.window, fast=rt.fast_kernels)
         a = torch.empty((a_lat.shape[0], self.heads, self.vdim), dtype=rt.act_dtype, device=a_lat.device)
         gate = pre[:, self.g_off:self.g_off + self.heads * self.vdim]
-        ops.head_product(a_lat, self.uv, a, gate=gate)
+        ops.head_product(a_lat, self.uv, a, gate=gate, fast=rt.fast_kernels)
         return self.out.add_into(a.view(a.shape[0], -1), x, then_norm, rt.act_dtype, scale=self.out_scale)

@@ -484,18 +484,48 @@ def test_one_key_stands_out(dtype, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_head_products_and_activation_alone(dtype):
+@pytest.mark.parametrize("rows, heads, n_in, n_out", [(37, 3, 20, 45), (100, 2, 24, 72), (5, 17, 128, 40), (300, 1, 8, 200)])
+def test_head_products_and_activation_alone(dtype, rows, heads, n_in, n_out):
+    """The per-head products, plain and (bfloat16, inner sizes in eights) on the matrix cores: into a
+    wider output of which only a head's own numbers may be written, with and without the gate."""
     from sonicboom_amd import ops
     dt = TORCH_DT[dtype]
-    x, w = rand(37, 3, 20).to(dt), rand(3, 20, 45, scale=0.3).to(dt)
-    out = torch.zeros((37, 3, 50), dtype=dt, device=DEV)
-    gate = rand(37, 200, seed=4).to(DEV)
-    ops.head_product(x.to(DEV), w.to(DEV), out, gate=gate[:, 10:10 + 135])
-    want = np.einsum("tai,aio->tao", x.float().numpy().astype(np.float64), w.float().numpy().astype(np.float64))
-    want = want * R.sigmoid(gate[:, 10:145].cpu().numpy().reshape(37, 3, 45))
-    part_close(out[:, :, :45], want, dtype, "head product")
-    assert float(out[:, :, 45:].abs().max()) == 0.0        # only a head's own numbers are written
+    x, w = rand(rows, heads, n_in).to(dt), rand(heads, n_out, n_in, scale=0.3).to(dt)
+    gate = rand(rows, heads * n_out + 16, seed=4).to(DEV)
+    want = np.einsum("tai,aoi->tao", x.float().numpy().astype(np.float64), w.float().numpy().astype(np.float64))
+    for g in (None, gate[:, 8:8 + heads * n_out]):
+        out = torch.zeros((rows, heads, n_out + 8), dtype=dt, device=DEV)
+        ops.head_product(x.to(DEV), w.to(DEV), out, gate=g)
+        ref = want if g is None else want * R.sigmoid(g.cpu().numpy().reshape(rows, heads, n_out))
+        part_close(out[:, :, :n_out], ref, dtype, "head product")
+        assert float(out[:, :, n_out:].abs().max()) == 0.0        # only a head's own numbers are written
     z = torch.linspace(-9, 9, 400)
     p = torch.tensor([0.4, -0.3]).to(dt)
     got = ops.activate(z.to(DEV), dt, "xielu", p.to(DEV))
     part_close(got, R.xielu(z.numpy(), float(p[0]), float(p[1])), dtype, "xielu")
+
+
+@pytest.mark.parametrize("heads, dim, rot_dim, vdim, rank, window", [
+    (4, 32, 16, 24, 64, 0), (20, 16, 8, 16, 40, 100), (3, 64, 32, 40, 256, 70), (2, 128, 64, 128, 512, 130)])
+def test_matrix_core_latent_attention_equals_the_plain_kernel(heads, dim, rot_dim, vdim, rank, window):
+    """bfloat16, the sizes of each compiled shape of the matrix-core kernel: a prompt, portions, and
+    single rows (where a wave takes 16 heads of a row) against the kernel of one wave per (row, head)."""
+    from sonicboom_amd.parts import build_part
+    from sonicboom_amd.parts.latent_attention import latent_attention_spec
+    from sonicboom_amd.parts.position import rope_interleaved_spec
+    from sonicboom_amd.parts import Runtime
+    width, n = 64, 330
+    spec = latent_attention_spec("a.", width, heads, dim, rot_dim, vdim, rank, 0.5, rope_interleaved_spec(rot_dim, 1e4),
+                                 window=window, eps=1e-5)
+    dev, ref = part_tensors(spec, "bfloat16", scale=0.5)
+    h = rand(n, width).to(BF16)
+    outs = {}
+    for fast in (True, False):
+        rt = Runtime(torch.device(DEV), BF16, fast)
+        mixer = build_part(spec, dict(dev), rt)
+        assert (getattr(mixer, "row_tile", None) is not None) == fast
+        feed = mixer_harness(mixer, rt)
+        outs[fast] = [feed(h, cuts, width) for cuts in ([n], [200, 66] + [1] * 64)]
+    for a, b in zip(outs[True], outs[False]):
+        part_close(a, b.float().cpu().numpy(), "bfloat16", "matrix-core against plain")
+    part_close(outs[True][1], outs[True][0].float().cpu().numpy(), "bfloat16", "portions and single rows against whole")
