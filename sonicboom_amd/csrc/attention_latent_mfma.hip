@@ -8,12 +8,13 @@
 //
 // sb_latent_attention_bf16: all query heads read the same cached rows [c | r], so a block stages
 // a page of 64 rows once in LDS, twice over: as it lies (a key's numbers consecutive: the A
-// operand of S^T = K Q^T) and with the latent part turned (a number's 64 keys consecutive: the A
-// operand of O^T = C^T P^T), and its four waves each run a tile of 16 query columns against it.
+// operand of S^T = K Q^T) and with the latent part turned (a number's keys consecutive: the A
+// operand of O^T = C^T P^T), half a page at a time in two buffers that take turns, and its four
+// waves each run a tile of 16 query columns against it.
 // In a prompt step a wave's 16 columns are 16 consecutive rows of one head; in a decode step they
-// are 16 heads of the one row.  The next page's rows are asked of memory before the current
-// page's products start and wait in registers.  Softmax runs in the result layout of S^T (a lane
-// holds 16 keys of one column a page; column maximum and sum over the four lane groups), P goes
+// are 16 heads of the one row.  The next half's rows are asked of memory before the current
+// half's products start, wait in registers and go into the other buffer afterwards.  Softmax runs
+// in the result layout of S^T (a lane holds 8 keys of one column; column maximum and sum over the four lane groups), P goes
 // back in as the B operand of the second product without leaving registers: the keys of a
 // 32-key step are taken in the order the first product left them, by V's fragment reads.
 #include "mfma.h"
@@ -23,7 +24,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kPadK = 8;     // bf16 a key row is padded by in LDS
-constexpr int kVtStride = SB_PAGE + 8;
+constexpr int kHalf = 32;    // keys of a step
+constexpr int kVtStride = kHalf + 8;
+constexpr float kLazy = 8.0f;   // how far (in powers of two) a score may pass the running maximum before it moves
 
 template <bool GATED>
 __global__ void __launch_bounds__(kThreads)
@@ -69,18 +72,23 @@ head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstri
 }
 
 // KQ: steps of 32 over a latent row that the unrolled loops cover; NV: tiles of 16 over the latent part.
+// A page is worked on in two halves of kHalf keys; LDS holds two halves at a time (the one the
+// waves read and the one being written), each as key rows [kHalf][lk] and as turned latent rows
+// [nv * 16][kVtStride].
 template <int KQ, int NV>
 __global__ void __launch_bounds__(kThreads)
 latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, const bf16_t *__restrict__ cache,
                              const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                              const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles, int heads, int rank,
-                             int rot_dim, float scale, int window, int tile_rows) {
+                             int rot_dim, float scale, int window, int tile_rows, int n_splits,
+                             float *__restrict__ part_o, float *__restrict__ part_ml, int n_rows) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int latent = rank + rot_dim;
   const int kq = (latent + 31) / 32, nv = (rank + 15) / 16;
   const int lk = kq * 32 + kPadK;                    // bf16 per staged key row
-  bf16_t *ks = reinterpret_cast<bf16_t *>(lds);      // [SB_PAGE][lk]
-  bf16_t *vt = ks + SB_PAGE * lk;                    // [nv * 16][kVtStride]
+  const int ks_size = kHalf * lk, vt_size = nv * 16 * kVtStride;
+  bf16_t *ks_base = reinterpret_cast<bf16_t *>(lds); // [2][kHalf][lk]
+  bf16_t *vt_base = ks_base + 2 * ks_size;           // [2][nv * 16][kVtStride]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, g = lane >> 4;
   const int r0 = tiles[4 * blockIdx.x], n_tile = tiles[4 * blockIdx.x + 1], seq = tiles[4 * blockIdx.x + 2];
@@ -97,15 +105,12 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   const int hi_blk = pos0 + n_tile - 1;
 
   // the pads that staging never writes must not hold what multiplies to NaN
-  for (int i = tid; i < SB_PAGE * (lk - latent); i += kThreads) {
+  for (int i = tid; i < 2 * kHalf * (lk - latent); i += kThreads) {
     const int key = i / (lk - latent), e = i - key * (lk - latent);
-    ks[key * lk + latent + e] = 0;
+    ks_base[key * lk + latent + e] = 0;
   }
-  for (int i = tid; i < (nv * 16 - rank) * kVtStride; i += kThreads) vt[rank * kVtStride + i] = 0;
-  for (int i = tid; i < rank * (kVtStride - SB_PAGE); i += kThreads) {
-    const int d = i / (kVtStride - SB_PAGE), e = i - d * (kVtStride - SB_PAGE);
-    vt[d * kVtStride + SB_PAGE + e] = 0;
-  }
+  for (int b = 0; b < 2; ++b)
+    for (int i = tid; i < (nv * 16 - rank) * kVtStride; i += kThreads) vt_base[b * vt_size + rank * kVtStride + i] = 0;
 
   // this lane's query fragments: column (row, head), k = 32 kk + 8 g .. + 7
   uint4 qf[KQ];
@@ -117,119 +122,167 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   }
 
   const float neg_inf = -__builtin_inff();
+  const float scale2 = scale * 1.4426950408889634f;     // scores in units of ln 2: the weights are exp2
   float m_run = neg_inf, l_run = 0.0f;
   floatx4_t o[NV];
 #pragma unroll
   for (int v = 0; v < NV; ++v) o[v] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  // staging: a page is 64 rows of latent / 8 chunks of 16 bytes; thread (key = idx % 64, chunk = idx / 64)
+  // staging: a half is kHalf rows of latent / 8 chunks of 16 bytes; thread (key = idx % kHalf, chunk = idx / kHalf)
   const int chunks = latent / 8;
-  constexpr int kMaxStage = (KQ * 32 / 8 * SB_PAGE + kThreads - 1) / kThreads;
+  constexpr int kMaxStage = (KQ * 32 / 8 * kHalf + kThreads - 1) / kThreads;
   uint4 staged[kMaxStage];
-  const int c_first = lo_blk / SB_PAGE, c_last = hi_blk / SB_PAGE;
-  auto page_of = [&](int c) -> int {
+  int h_first = lo_blk / kHalf, h_last = hi_blk / kHalf;                // halves count from the sequence's start
+  if (n_splits > 1) {                                                   // this block's share of them
+    const int per = (h_last - h_first + n_splits) / n_splits;
+    h_first += int(blockIdx.z) * per;
+    h_last = min(h_last, h_first + per - 1);
+  }
+  auto page_of = [&](int h) -> int {
+    const int c = h / (SB_PAGE / kHalf);
     const int p = c < max_pages ? page_table[size_t(seq) * max_pages + c] : -1;
     return (p >= 0 && p < n_pages_total) ? p : -1;
   };
-  auto load_page = [&](int page) {
+  auto load_half = [&](int h) {
+    const int page = page_of(h);
+    const bf16_t *src = cache + (size_t(max(page, 0)) * SB_PAGE + (h % (SB_PAGE / kHalf)) * kHalf) * latent;
 #pragma unroll
     for (int it = 0; it < kMaxStage; ++it) {
       const int idx = tid + it * kThreads;
-      const int key = idx & 63, chunk = idx >> 6;
-      staged[it] = ld16(cache + (size_t(max(page, 0)) * SB_PAGE + key) * latent + 8 * min(chunk, chunks - 1),
-                        page >= 0 && chunk < chunks);
+      const int key = idx % kHalf, chunk = idx / kHalf;
+      staged[it] = ld16(src + size_t(key) * latent + 8 * min(chunk, chunks - 1), page >= 0 && chunk < chunks);
     }
   };
-  auto store_page = [&]() {
+  // A thread holds eight numbers of one key; the turned copy wants a number's keys side by side.
+  // Neighbouring lanes hold neighbouring keys of the same chunk, so a pair of lanes swaps half of
+  // what it holds (two DPP moves inside the quad) and each writes four whole 32-bit words, (even
+  // key, odd key) of one number each: the even lane numbers 0 to 3 of the chunk, the odd lane 4 to 7.
+  // (Written as single 16-bit stores, two lanes a word, this step took as long as all the products.)
+  auto store_half = [&](int b) {
+    bf16_t *ks = ks_base + b * ks_size;
+    uint32_t *vt32 = reinterpret_cast<uint32_t *>(vt_base + b * vt_size);
+    const bool even = (lane & 1) == 0;
 #pragma unroll
     for (int it = 0; it < kMaxStage; ++it) {
       const int idx = tid + it * kThreads;
-      const int key = idx & 63, chunk = idx >> 6;
+      const int key = idx % kHalf, chunk = idx / kHalf;
+      const uint4 st = staged[it];
+      const uint32_t send0 = even ? st.z : st.x, send1 = even ? st.w : st.y;
+      const uint32_t recv0 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send0), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+      const uint32_t recv1 = uint32_t(__builtin_amdgcn_update_dpp(0, int(send1), 0xB1, 0xF, 0xF, true));
       if (chunk >= chunks) continue;
-      *reinterpret_cast<uint4 *>(ks + key * lk + 8 * chunk) = staged[it];
-      if (8 * chunk < rank) {
-        const uint32_t wds[4] = {staged[it].x, staged[it].y, staged[it].z, staged[it].w};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int d = 8 * chunk + e;
-          if (d < rank) vt[d * kVtStride + key] = bf16_t((wds[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-        }
+      *reinterpret_cast<uint4 *>(ks + key * lk + 8 * chunk) = st;
+      if (8 * chunk < rank) {                       // rank is a multiple of 8: a chunk lies inside or outside
+        const uint32_t mine0 = even ? st.x : st.z, mine1 = even ? st.y : st.w;
+        const uint32_t lo0 = even ? mine0 : recv0, hi0 = even ? recv0 : mine0;   // the even key's numbers, the odd key's
+        const uint32_t lo1 = even ? mine1 : recv1, hi1 = even ? recv1 : mine1;
+        const int d = 8 * chunk + (even ? 0 : 4);
+        uint32_t *dst = vt32 + (d * kVtStride + (key & ~1)) / 2;
+        dst[0 * (kVtStride / 2)] = (lo0 & 0xffffu) | (hi0 << 16);
+        dst[1 * (kVtStride / 2)] = (lo0 >> 16) | (hi0 & 0xffff0000u);
+        dst[2 * (kVtStride / 2)] = (lo1 & 0xffffu) | (hi1 << 16);
+        dst[3 * (kVtStride / 2)] = (lo1 >> 16) | (hi1 & 0xffff0000u);
       }
     }
   };
 
-  int c = c_first;
-  while (c <= c_last && page_of(c) < 0) ++c;          // pages that are not there hold no visible key
-  if (c <= c_last) load_page(page_of(c));
-  while (c <= c_last) {
-    __syncthreads();                                  // the page before has been read by every wave
-    store_page();
-    __syncthreads();
-    int c_next = c + 1;
-    while (c_next <= c_last && page_of(c_next) < 0) ++c_next;
-    if (c_next <= c_last) load_page(page_of(c_next)); // in flight while this page is worked on
+  int h = h_first;
+  while (h <= h_last && page_of(h) < 0) ++h;          // pages that are not there hold no visible key
+  int buf = 0;
+  if (h <= h_last) {
+    load_half(h);
+    store_half(0);
+  }
+  __syncthreads();                                    // the pads and the first half are written
+  while (h <= h_last) {
+    int h_next = h + 1;
+    while (h_next <= h_last && page_of(h_next) < 0) ++h_next;
+    if (h_next <= h_last) load_half(h_next);          // in flight while this half is worked on
 
     if (wave_works) {
-      floatx4_t s[4];
+      const bf16_t *ks = ks_base + buf * ks_size, *vt = vt_base + buf * vt_size;
+      floatx4_t s[2] = {floatx4_t{0.f, 0.f, 0.f, 0.f}, floatx4_t{0.f, 0.f, 0.f, 0.f}};
+      const bf16_t *kr = ks + col * lk + 8 * g;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-        const bf16_t *kr = ks + (16 * t + col) * lk + 8 * g;
+      for (int kk = 0; kk < KQ; ++kk) {
+        if (kk >= kq) continue;
 #pragma unroll
-        for (int kk = 0; kk < KQ; ++kk)
-          if (kk < kq) s[t] = mfma16(as_bf16x8(*reinterpret_cast<const uint4 *>(kr + 32 * kk)), as_bf16x8(qf[kk]), s[t]);
+        for (int t = 0; t < 2; ++t)
+          s[t] = mfma16(as_bf16x8(*reinterpret_cast<const uint4 *>(kr + 16 * t * lk + 32 * kk)), as_bf16x8(qf[kk]), s[t]);
       }
-      // s[t][i] = score of key 64 c + 16 t + 4 g + i for this lane's column
+      // s[t][i] = score of key kHalf h + 16 t + 4 g + i for this lane's column, in units of ln 2
       float mx = neg_inf;
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int j = c * SB_PAGE + 16 * t + 4 * g + i;
+          const int j = h * kHalf + 16 * t + 4 * g + i;
           const bool vis = valid && j >= lo && j <= pos;
-          s[t][i] = vis ? s[t][i] * scale : neg_inf;
+          s[t][i] = vis ? s[t][i] * scale2 : neg_inf;
           mx = fmaxf(mx, s[t][i]);
         }
       mx = max_over_lane_groups(mx);
-      const float m_new = fmaxf(m_run, mx);
-      const float m_safe = m_new == neg_inf ? 0.0f : m_new;
-      const float alpha = expf(m_run - m_safe);        // 0 while nothing has been seen
+      // the maximum the sums are relative to moves only when a score passes it by kLazy (2^kLazy in
+      // the weights, which float32 sums and bfloat16 weights carry easily): most steps then leave
+      // the accumulators alone
+      if (__any(mx > m_run + kLazy)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = m_new == neg_inf ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);   // 0 while nothing has been seen
+        l_run *= alpha;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[v][i] *= alpha;
+        m_run = m_new;
+      }
+      const float m_safe = m_run == neg_inf ? 0.0f : m_run;
       float sum = 0.0f;
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          s[t][i] = expf(s[t][i] - m_safe);
+          s[t][i] = __builtin_amdgcn_exp2f(s[t][i] - m_safe);
           sum += s[t][i];
         }
-      l_run = l_run * alpha + sum;
-      m_run = m_new;
-      uint4 pf[2];
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-        pf[u] = make_uint4(pack_bf16(s[2 * u][0], s[2 * u][1]), pack_bf16(s[2 * u][2], s[2 * u][3]),
-                           pack_bf16(s[2 * u + 1][0], s[2 * u + 1][1]), pack_bf16(s[2 * u + 1][2], s[2 * u + 1][3]));
+      l_run += sum;
+      const uint4 pf = make_uint4(pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
+                                  pack_bf16(s[1][0], s[1][1]), pack_bf16(s[1][2], s[1][3]));
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
         if (v >= nv) continue;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[v][i] *= alpha;
         const bf16_t *vr = vt + (16 * v + col) * kVtStride + 4 * g;
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const uint2 lo8 = *reinterpret_cast<const uint2 *>(vr + 32 * u);
-          const uint2 hi8 = *reinterpret_cast<const uint2 *>(vr + 32 * u + 16);
-          o[v] = mfma16(as_bf16x8(make_uint4(lo8.x, lo8.y, hi8.x, hi8.y)), as_bf16x8(pf[u]), o[v]);
-        }
+        const uint2 lo8 = *reinterpret_cast<const uint2 *>(vr);
+        const uint2 hi8 = *reinterpret_cast<const uint2 *>(vr + 16);
+        o[v] = mfma16(as_bf16x8(make_uint4(lo8.x, lo8.y, hi8.x, hi8.y)), as_bf16x8(pf), o[v]);
       }
     }
-    c = c_next;
+    // nobody reads the other buffer any more: its readers passed the barrier that ended the step before
+    if (h_next <= h_last) store_half(buf ^ 1);
+    __syncthreads();                                  // (after the stores: the loads they wait for have had the step's products to land)
+    buf ^= 1;
+    h = h_next;
   }
 
   if (!wave_works) return;
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
   l_tot += __shfl_xor(l_tot, 32, 64);
   if (!valid) return;
+  if (n_splits > 1) {               // unnormalized sums, with the maximum they are relative to, for the merge
+    const size_t column = size_t(blockIdx.z) * n_rows * heads + size_t(row) * heads + head;
+    float *po = part_o + column * rank;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      if (v >= nv) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (16 * v + 4 * g + i < rank) po[16 * v + 4 * g + i] = o[v][i];
+    }
+    if (g == 0) {
+      part_ml[2 * column] = m_run;
+      part_ml[2 * column + 1] = l_tot;
+    }
+    return;
+  }
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   bf16_t *orow = out + (size_t(row) * heads + head) * rank;
 #pragma unroll
@@ -247,13 +300,38 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   }
 }
 
+// out[column, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M the largest m_s: the shares of
+// a column's keys that n_splits blocks worked on, put together.  A block a column.
+__global__ void __launch_bounds__(256)
+latent_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                    int n_splits, size_t n_columns, int rank) {
+  const size_t column = blockIdx.x;
+  float m = -__builtin_inff();
+  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[2 * (size_t(s) * n_columns + column)]);
+  float l = 0.0f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float ms = part_ml[2 * (size_t(s) * n_columns + column)];
+    if (ms > -__builtin_inff()) l += part_ml[2 * (size_t(s) * n_columns + column) + 1] * exp2f(ms - m);
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  for (int d = threadIdx.x; d < rank; d += 256) {
+    float acc = 0.0f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float ms = part_ml[2 * (size_t(s) * n_columns + column)];
+      if (ms > -__builtin_inff()) acc += part_o[(size_t(s) * n_columns + column) * rank + d] * exp2f(ms - m);
+    }
+    out[column * rank + d] = f32_to_bf16(acc * inv);
+  }
+}
+
 template <int KQ, int NV>
 int launch_attention(bf16_t *out, const bf16_t *q, const bf16_t *cache, const int32_t *page_table, int max_pages,
                      int n_pages_total, const int32_t *row_pos, const int32_t *tiles, int n_tiles, int heads, int rank,
-                     int rot_dim, float scale, int window, int tile_rows, hipStream_t s) {
+                     int rot_dim, float scale, int window, int tile_rows, int n_splits, float *part_o, float *part_ml,
+                     int n_rows, hipStream_t s) {
   const int latent = rank + rot_dim;
   const int kq = (latent + 31) / 32, nv = (rank + 15) / 16;
-  const size_t lds = (size_t(SB_PAGE) * (kq * 32 + kPadK) + size_t(nv) * 16 * kVtStride) * sizeof(bf16_t);
+  const size_t lds = 2 * (size_t(kHalf) * (kq * 32 + kPadK) + size_t(nv) * 16 * kVtStride) * sizeof(bf16_t);
   static bool raised = false;              // once per kernel of this shape: more dynamic LDS than the default allows
   if (!raised) {
     if (hipFuncSetAttribute((const void *)latent_attention_mfma_kernel<KQ, NV>,
@@ -262,10 +340,13 @@ int launch_attention(bf16_t *out, const bf16_t *q, const bf16_t *cache, const in
     raised = true;
   }
   const int heads_per_block = kWaves * (16 / tile_rows);
-  dim3 grid(n_tiles, (heads + heads_per_block - 1) / heads_per_block);
+  dim3 grid(n_tiles, (heads + heads_per_block - 1) / heads_per_block, n_splits);
   latent_attention_mfma_kernel<KQ, NV><<<grid, kThreads, lds, s>>>(out, q, cache, page_table, max_pages, n_pages_total,
                                                                    row_pos, tiles, heads, rank, rot_dim, scale, window,
-                                                                   tile_rows);
+                                                                   tile_rows, n_splits, part_o, part_ml, n_rows);
+  if (n_splits > 1)
+    latent_merge_kernel<<<unsigned(size_t(n_rows) * heads), 256, 0, s>>>(out, part_o, part_ml, n_splits,
+                                                                         size_t(n_rows) * heads, rank);
   return sb::check_launch("sb_latent_attention_bf16");
 }
 
@@ -315,14 +396,20 @@ extern "C" int sb_latent_attention_bf16_ok(int rank, int rot_dim) {
 // file).  tiles int32 [n_tiles, 4] = (first row, rows, sequence, 0): runs of up to tile_rows
 // consecutive rows of one sequence; tile_rows 16 for a prompt step, 1 for a step of single rows
 // (a wave then takes 16 heads of a row).  out [n_rows, heads, rank], q [n_rows, heads, rank + rot_dim].
+// n_splits > 1: the keys of every tile are shared out over that many blocks, whose unnormalized sums
+// go through part_o (f32 [n_splits, n_rows, heads, rank]) and part_ml (f32 [n_splits, n_rows, heads, 2])
+// and are put together by a second kernel: for steps of few rows over many keys.
 extern "C" int sb_latent_attention_bf16(void *out, const void *q, const void *cache, const int32_t *page_table,
                                         int max_pages, int n_pages_total, const int32_t *row_pos, const int32_t *tiles,
                                         int n_tiles, int heads, int rank, int rot_dim, float scale, int window,
-                                        int tile_rows, void *stream) {
+                                        int tile_rows, int n_splits, float *part_o, float *part_ml, int n_rows,
+                                        void *stream) {
   SB_REQUIRE(out && q && cache && page_table && row_pos && tiles, "sb_latent_attention_bf16: null pointer");
   SB_REQUIRE(n_tiles >= 0 && heads > 0 && max_pages > 0 && n_pages_total > 0 && window >= 0,
              "sb_latent_attention_bf16: bad sizes");
   SB_REQUIRE(tile_rows == 16 || tile_rows == 1, "sb_latent_attention_bf16: tiles of 16 rows or of one");
+  SB_REQUIRE(n_splits >= 1 && n_splits <= 65535 && n_rows >= 0 && (n_splits == 1 || (part_o && part_ml)),
+             "sb_latent_attention_bf16: shares of the keys need their scratch");
   SB_SUPPORT(sb_latent_attention_bf16_ok(rank, rot_dim), "sb_latent_attention_bf16: a latent row of %d + %d is not taken",
              rank, rot_dim);
   SB_SUPPORT((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(cache) | reinterpret_cast<uintptr_t>(out)) % 16 == 0,
@@ -332,7 +419,8 @@ extern "C" int sb_latent_attention_bf16(void *out, const void *q, const void *ca
   const int kq = (rank + rot_dim + 31) / 32, nv = (rank + 15) / 16;
 #define SB_GO(KQ, NV)                                                                                              \
   return launch_attention<KQ, NV>((bf16_t *)out, (const bf16_t *)q, (const bf16_t *)cache, page_table, max_pages,    \
-                                  n_pages_total, row_pos, tiles, n_tiles, heads, rank, rot_dim, scale, window, tile_rows, s)
+                                  n_pages_total, row_pos, tiles, n_tiles, heads, rank, rot_dim, scale, window, tile_rows,  \
+                                  n_splits, part_o, part_ml, n_rows, s)
   if (kq <= 6 && nv <= 8) SB_GO(6, 8);
   if (kq <= 10 && nv <= 16) SB_GO(10, 16);
   SB_GO(18, 32);

@@ -216,7 +216,9 @@ int sb_latent_attention(void *out, const void *q, int act_dtype, const void *cac
 /* The same two on the matrix cores, everything bfloat16 (csrc/attention_latent_mfma.hip); the
  * *_ok functions say whether the sizes are taken.  tiles int32 [n_tiles, 4] = (first row, rows,
  * sequence, 0): runs of up to tile_rows consecutive rows of a sequence, tile_rows 16 (a wave takes 16
- * rows of a head) or 1 (16 heads of a row). */
+ * rows of a head) or 1 (16 heads of a row).  n_splits > 1: every tile's keys are shared out over that
+ * many blocks and put together by a second kernel, through part_o f32 [n_splits, n_rows, heads, rank]
+ * and part_ml f32 [n_splits, n_rows, heads, 2]. */
 int sb_head_product_bf16_ok(int out_stride, int out_hstride, int in_stride, int in_hstride, int n_in);
 int sb_head_product_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride,
                          int in_hstride, const void *w, const float *gate, int gate_stride, int n_rows,
@@ -226,7 +228,7 @@ int sb_latent_attention_bf16_ok(int rank, int rot_dim);
 int sb_latent_attention_bf16(void *out, const void *q, const void *cache, const int32_t *page_table,
                              int max_pages, int n_pages_total, const int32_t *row_pos, const int32_t *tiles,
                              int n_tiles, int heads, int rank, int rot_dim, float scale, int window,
-                             int tile_rows, void *stream);
+                             int tile_rows, int n_splits, float *part_o, float *part_ml, int n_rows, void *stream);
 
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts

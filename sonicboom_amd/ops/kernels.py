@@ -980,10 +980,17 @@ def latent_attention_mfma_ok(q_dtype, cache_dtype, rank: int, rot_dim: int) -> b
         and bool(library.core().sb_latent_attention_bf16_ok(int(rank), int(rot_dim)))
 
 
+LATENT_SPLIT_BLOCKS = 512       # blocks a step of few rows aims at by sharing out its keys
+LATENT_SPLIT_KEYS = 64          # keys a share has at least
+
+
 def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, row_pos: torch.Tensor,
-                          tiles: torch.Tensor, rank: int, scale: float, window: int, single_rows: bool) -> torch.Tensor:
+                          tiles: torch.Tensor, rank: int, scale: float, window: int, single_rows: bool,
+                          max_keys: int = 0) -> torch.Tensor:
     """The matrix-core form: ``tiles`` int32 [n, 4], runs of up to 16 consecutive rows of a sequence;
-    ``single_rows``: every run is one row (a decode step), a wave then takes 16 heads of it."""
+    ``single_rows``: every run is one row (a decode step), a wave then takes 16 heads of it.
+    ``max_keys`` (the most keys a row of the step sees, if the caller knows): a launch of few blocks
+    over many keys shares the keys of every run out over several blocks and merges their results."""
     _dev(q, cache, page_table, row_pos, tiles)
     n, heads, latent = q.shape
     if cache.dim() != 3 or cache.shape[1] != PAGE or cache.shape[2] != latent:
@@ -994,10 +1001,18 @@ def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, page_table: torc
     if page_table.dtype != torch.int32 or page_table.dim() != 2:
         raise KernelLibraryError("the page table must be int32 [sequences, pages]")
     out = torch.empty((n, heads, rank), dtype=q.dtype, device=q.device)
+    blocks = tiles.shape[0] * -(-heads // (64 if single_rows else 4))
+    splits = 1
+    if max_keys > LATENT_SPLIT_KEYS and 0 < blocks < LATENT_SPLIT_BLOCKS:
+        splits = max(1, min(-(-LATENT_SPLIT_BLOCKS // blocks), max_keys // LATENT_SPLIT_KEYS))
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((splits, n, heads, rank), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((splits, n, heads, 2), dtype=torch.float32, device=q.device)
     check(library.core().sb_latent_attention_bf16(_p(out), _p(q), _p(cache), _p(page_table), page_table.shape[1],
                                                   cache.shape[0], _p(row_pos), _p(tiles), tiles.shape[0], heads, rank,
                                                   latent - rank, float(scale), int(window), 1 if single_rows else 16,
-                                                  _stream()))
+                                                  splits, _p(part_o), _p(part_ml), n, _stream()))
     return out
 
 
@@ -1007,6 +1022,8 @@ def latent_attention(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Ten
     types (the step's context then lists the rows in runs of LATENT_ROW_TILE), else the kernel of
     one wave per (row, head)."""
     if fast and latent_attention_mfma_ok(q.dtype, cache.dtype, rank, q.shape[2] - rank):
+        keys = int(getattr(ctx, "max_len_after", 0) or 0)
         return latent_attention_mfma(q, cache, page_table, ctx.row_pos, ctx.row_tiles(LATENT_ROW_TILE), rank, scale,
-                                     window, single_rows=bool(ctx.is_decode))
+                                     window, single_rows=bool(ctx.is_decode),
+                                     max_keys=min(keys, window) if window > 0 else keys)
     return latent_attention_plain(q, cache, page_table, ctx.row_pos, ctx.row_seq, rank, scale, window)

@@ -52,7 +52,7 @@ _CORE_SIGNATURES = {
     "sb_head_product_bf16": [_P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "sb_latent_attention_tile_rows": [],
     "sb_latent_attention_bf16_ok": [_I, _I],
-    "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
+    "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {
