@@ -9,8 +9,8 @@
 // sb_latent_attention_bf16: all query heads read the same cached rows [c | r], so a block stages
 // a page of 64 rows once in LDS, twice over: as it lies (a key's numbers consecutive: the A
 // operand of S^T = K Q^T) and with the latent part turned (a number's keys consecutive: the A
-// operand of O^T = C^T P^T), half a page at a time in two buffers that take turns, and its four
-// waves each run a tile of 16 query columns against it.
+// operand of O^T = C^T P^T), half a page at a time in two buffers that take turns, and its eight
+// waves run four tiles of 16 query columns against it, two waves a tile.
 // In a prompt step a wave's 16 columns are 16 consecutive rows of one head; in a decode step they
 // are 16 heads of the one row.  The next half's rows are asked of memory before the current
 // half's products start, wait in registers and go into the other buffer afterwards.  Softmax runs
@@ -21,8 +21,10 @@
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
+constexpr int kThreads = 256;      // of the per-head product
+constexpr int kAttnThreads = 512;  // of attention: eight waves,
+constexpr int kColGroups = 4;      // four tiles of 16 query columns,
+constexpr int kParts = 2;          // two waves a tile
 constexpr int kPadK = 8;     // bf16 a key row is padded by in LDS
 constexpr int kHalf = 32;    // keys of a step
 constexpr int kVtStride = kHalf + 8;
@@ -74,9 +76,11 @@ head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstri
 // KQ: steps of 32 over a latent row that the unrolled loops cover; NV: tiles of 16 over the latent part.
 // A page is worked on in two halves of kHalf keys; LDS holds two halves at a time (the one the
 // waves read and the one being written), each as key rows [kHalf][lk] and as turned latent rows
-// [nv * 16][kVtStride].
+// [nv * 16][kVtStride].  Eight waves: a tile of 16 query columns belongs to two waves, which both
+// work out its scores and weights and take half of the latent part's tiles each in the second
+// product, so that a wave's accumulators and fragments leave room for two waves a SIMD.
 template <int KQ, int NV>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kAttnThreads)
 latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, const bf16_t *__restrict__ cache,
                              const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                              const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles, int heads, int rank,
@@ -91,11 +95,15 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   bf16_t *vt_base = ks_base + 2 * ks_size;           // [2][nv * 16][kVtStride]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, g = lane >> 4;
-  const int r0 = tiles[4 * blockIdx.x], n_tile = tiles[4 * blockIdx.x + 1], seq = tiles[4 * blockIdx.x + 2];
+  // the last tiles of a prompt see the most keys: they go first, so that the short ones fill the end
+  const int tile = int(gridDim.x) - 1 - int(blockIdx.x);
+  const int r0 = tiles[4 * tile], n_tile = tiles[4 * tile + 1], seq = tiles[4 * tile + 2];
   const int heads_per_wave = 16 / tile_rows;
-  const int head = (blockIdx.y * kWaves + wave) * heads_per_wave + col / tile_rows;
+  const int group = wave / kParts, part = wave % kParts;       // the wave's tile of columns, and its share of the latent part
+  const int nv_part = (nv + kParts - 1) / kParts;
+  const int head = (blockIdx.y * kColGroups + group) * heads_per_wave + col / tile_rows;
   const int r = col % tile_rows;
-  const bool wave_works = (blockIdx.y * kWaves + wave) * heads_per_wave < heads;
+  const bool wave_works = (blockIdx.y * kColGroups + group) * heads_per_wave < heads;
   const bool valid = r < n_tile && head < heads;
   const int row = r0 + min(r, n_tile - 1);
   const int pos0 = row_pos[r0];
@@ -105,12 +113,12 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   const int hi_blk = pos0 + n_tile - 1;
 
   // the pads that staging never writes must not hold what multiplies to NaN
-  for (int i = tid; i < 2 * kHalf * (lk - latent); i += kThreads) {
+  for (int i = tid; i < 2 * kHalf * (lk - latent); i += kAttnThreads) {
     const int key = i / (lk - latent), e = i - key * (lk - latent);
     ks_base[key * lk + latent + e] = 0;
   }
   for (int b = 0; b < 2; ++b)
-    for (int i = tid; i < (nv * 16 - rank) * kVtStride; i += kThreads) vt_base[b * vt_size + rank * kVtStride + i] = 0;
+    for (int i = tid; i < (nv * 16 - rank) * kVtStride; i += kAttnThreads) vt_base[b * vt_size + rank * kVtStride + i] = 0;
 
   // this lane's query fragments: column (row, head), k = 32 kk + 8 g .. + 7
   uint4 qf[KQ];
@@ -124,13 +132,14 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   const float neg_inf = -__builtin_inff();
   const float scale2 = scale * 1.4426950408889634f;     // scores in units of ln 2: the weights are exp2
   float m_run = neg_inf, l_run = 0.0f;
-  floatx4_t o[NV];
+  constexpr int NVP = (NV + kParts - 1) / kParts;
+  floatx4_t o[NVP];
 #pragma unroll
-  for (int v = 0; v < NV; ++v) o[v] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int v = 0; v < NVP; ++v) o[v] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
   // staging: a half is kHalf rows of latent / 8 chunks of 16 bytes; thread (key = idx % kHalf, chunk = idx / kHalf)
   const int chunks = latent / 8;
-  constexpr int kMaxStage = (KQ * 32 / 8 * kHalf + kThreads - 1) / kThreads;
+  constexpr int kMaxStage = (KQ * 32 / 8 * kHalf + kAttnThreads - 1) / kAttnThreads;
   uint4 staged[kMaxStage];
   int h_first = lo_blk / kHalf, h_last = hi_blk / kHalf;                // halves count from the sequence's start
   if (n_splits > 1) {                                                   // this block's share of them
@@ -148,7 +157,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
     const bf16_t *src = cache + (size_t(max(page, 0)) * SB_PAGE + (h % (SB_PAGE / kHalf)) * kHalf) * latent;
 #pragma unroll
     for (int it = 0; it < kMaxStage; ++it) {
-      const int idx = tid + it * kThreads;
+      const int idx = tid + it * kAttnThreads;
       const int key = idx % kHalf, chunk = idx / kHalf;
       staged[it] = ld16(src + size_t(key) * latent + 8 * min(chunk, chunks - 1), page >= 0 && chunk < chunks);
     }
@@ -164,7 +173,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
     const bool even = (lane & 1) == 0;
 #pragma unroll
     for (int it = 0; it < kMaxStage; ++it) {
-      const int idx = tid + it * kThreads;
+      const int idx = tid + it * kAttnThreads;
       const int key = idx % kHalf, chunk = idx / kHalf;
       const uint4 st = staged[it];
       const uint32_t send0 = even ? st.z : st.x, send1 = even ? st.w : st.y;
@@ -230,7 +239,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
         const float alpha = m_new == neg_inf ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);   // 0 while nothing has been seen
         l_run *= alpha;
 #pragma unroll
-        for (int v = 0; v < NV; ++v)
+        for (int v = 0; v < NVP; ++v)
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[v][i] *= alpha;
         m_run = m_new;
@@ -248,9 +257,10 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
       const uint4 pf = make_uint4(pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]),
                                   pack_bf16(s[1][0], s[1][1]), pack_bf16(s[1][2], s[1][3]));
 #pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        if (v >= nv) continue;
-        const bf16_t *vr = vt + (16 * v + col) * kVtStride + 4 * g;
+      for (int v = 0; v < NVP; ++v) {
+        const int vg = part * nv_part + v;
+        if (v >= nv_part || vg >= nv) continue;
+        const bf16_t *vr = vt + (16 * vg + col) * kVtStride + 4 * g;
         const uint2 lo8 = *reinterpret_cast<const uint2 *>(vr);
         const uint2 hi8 = *reinterpret_cast<const uint2 *>(vr + 16);
         o[v] = mfma16(as_bf16x8(make_uint4(lo8.x, lo8.y, hi8.x, hi8.y)), as_bf16x8(pf), o[v]);
@@ -271,13 +281,14 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
     const size_t column = size_t(blockIdx.z) * n_rows * heads + size_t(row) * heads + head;
     float *po = part_o + column * rank;
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      if (v >= nv) continue;
+    for (int v = 0; v < NVP; ++v) {
+      const int vg = part * nv_part + v;
+      if (v >= nv_part || vg >= nv) continue;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (16 * v + 4 * g + i < rank) po[16 * v + 4 * g + i] = o[v][i];
+        if (16 * vg + 4 * g + i < rank) po[16 * vg + 4 * g + i] = o[v][i];
     }
-    if (g == 0) {
+    if (g == 0 && part == 0) {
       part_ml[2 * column] = m_run;
       part_ml[2 * column + 1] = l_tot;
     }
@@ -286,9 +297,10 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   bf16_t *orow = out + (size_t(row) * heads + head) * rank;
 #pragma unroll
-  for (int v = 0; v < NV; ++v) {
-    if (v >= nv) continue;
-    const int d = 16 * v + 4 * g;
+  for (int v = 0; v < NVP; ++v) {
+    const int vg = part * nv_part + v;
+    if (v >= nv_part || vg >= nv) continue;
+    const int d = 16 * vg + 4 * g;
     if (d + 3 < rank) {
       *reinterpret_cast<uint2 *>(orow + d) = make_uint2(pack_bf16(o[v][0] * inv, o[v][1] * inv),
                                                         pack_bf16(o[v][2] * inv, o[v][3] * inv));
@@ -339,9 +351,9 @@ int launch_attention(bf16_t *out, const bf16_t *q, const bf16_t *cache, const in
       (void)hipGetLastError();
     raised = true;
   }
-  const int heads_per_block = kWaves * (16 / tile_rows);
+  const int heads_per_block = kColGroups * (16 / tile_rows);
   dim3 grid(n_tiles, (heads + heads_per_block - 1) / heads_per_block, n_splits);
-  latent_attention_mfma_kernel<KQ, NV><<<grid, kThreads, lds, s>>>(out, q, cache, page_table, max_pages, n_pages_total,
+  latent_attention_mfma_kernel<KQ, NV><<<grid, kAttnThreads, lds, s>>>(out, q, cache, page_table, max_pages, n_pages_total,
                                                                    row_pos, tiles, heads, rank, rot_dim, scale, window,
                                                                    tile_rows, n_splits, part_o, part_ml, n_rows);
   if (n_splits > 1)
