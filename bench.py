@@ -658,8 +658,8 @@ def rasizen_sizes(width, n_blocks=2, window=4096, vocab=32768):
             "norm": {"eps": 1e-5, "groups": 2}, "layers": layers}
 
 
-def qwen_sizes(width, n_layers=4, vocab=32768):
-    """The Qwen2.5 design at the same width and head count, a gated feed-forward of the same weight
+def qwen_sizes(width, n_layers=8, vocab=32768):
+    """The Qwen2.5 design at the same width, head count and number of layers, a gated feed-forward of the same weight
     count as the ungated one of 4 widths (inner 8/3 widths, in 256s), a quarter of the heads as kv heads."""
     heads = width // 128
     return dict(CONFIG_7B, num_hidden_layers=n_layers, hidden_size=width, num_attention_heads=heads,

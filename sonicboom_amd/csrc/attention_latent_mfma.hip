@@ -45,16 +45,24 @@ head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstri
   floatx4_t acc[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < n_in; k0 += 32) {
-    const int k = k0 + 8 * g;
-    const bool kin = k < n_in;                                   // n_in is a multiple of 8
-    const uint4 b = ld16(xin + (kin ? k : 0), kin && t < n_rows);
+  // four steps of 32 k at a time: their twenty loads go out together, then the sixteen products
+  for (int k0 = 0; k0 < n_in; k0 += 128) {
+    uint4 b[4], av[4][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int o = o0 + 16 * j + (lane & 15);
-      const uint4 av = ld16(wa + size_t(min(o, n_out - 1)) * n_in + (kin ? k : 0), kin && o < n_out);
-      acc[j] = mfma16(as_bf16x8(av), as_bf16x8(b), acc[j]);
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 32 * u + 8 * g;
+      const bool kin = k < n_in;                                 // n_in is a multiple of 8
+      b[u] = ld16(xin + (kin ? k : 0), kin && t < n_rows);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int o = o0 + 16 * j + (lane & 15);
+        av[u][j] = ld16(wa + size_t(min(o, n_out - 1)) * n_in + (kin ? k : 0), kin && o < n_out);
+      }
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = mfma16(as_bf16x8(av[u][j]), as_bf16x8(b[u]), acc[j]);
   }
   if (t >= n_rows) return;
 #pragma unroll

@@ -213,11 +213,37 @@ group_norm_kernel(TO *__restrict__ y, float *x, const int32_t *__restrict__ rows
   const int gw = width / groups;
   const int wpg = groups >= kGroupWaves ? 1 : kGroupWaves / groups;   // waves that share a group: 1, 2 or 4
   const int per_pass = kGroupWaves / wpg;                              // groups the block takes at a time
+  // four elements a lane at a time where the parts allow it (every part a multiple of four wide, the
+  // row on 16 bytes): the same sums in the same order per lane, only wider loads and stores
+  const bool vec = (gw % 4 == 0) && ((reinterpret_cast<uintptr_t>(xr) | reinterpret_cast<uintptr_t>(pr) |
+                                      (size_t(slice_stride) * 4)) % 16 == 0);
   for (int g0 = 0; g0 < groups; g0 += per_pass) {
     const int g = g0 + wave / wpg, k = wave % wpg;
     const bool active = g < groups;
     double part = 0.0;
-    if (active) {
+    if (active && vec) {
+      for (int i = 4 * (lane + 64 * k); i < gw; i += 256 * wpg) {
+        const size_t e = size_t(g) * gw + i;
+        float4 v;
+        if (pr) {
+          float4 acc = *reinterpret_cast<const float4 *>(pr + e);
+          for (int s = 1; s < n_slices; ++s) {
+            const float4 p4 = *reinterpret_cast<const float4 *>(pr + size_t(s) * slice_stride + e);
+            acc.x += p4.x; acc.y += p4.y; acc.z += p4.z; acc.w += p4.w;
+          }
+          if (bias) {
+            acc.x += ld_dyn(bias, bias_dtype, e); acc.y += ld_dyn(bias, bias_dtype, e + 1);
+            acc.z += ld_dyn(bias, bias_dtype, e + 2); acc.w += ld_dyn(bias, bias_dtype, e + 3);
+          }
+          const float4 old = *reinterpret_cast<const float4 *>(xr + e);
+          v = make_float4(acc.x * scale + old.x, acc.y * scale + old.y, acc.z * scale + old.z, acc.w * scale + old.w);
+          *reinterpret_cast<float4 *>(xr + e) = v;
+        } else {
+          v = *reinterpret_cast<const float4 *>(xr + e);
+        }
+        part += squares(v);
+      }
+    } else if (active) {
       for (int i = lane + 64 * k; i < gw; i += 64 * wpg) {
         const size_t e = size_t(g) * gw + i;
         float v;
@@ -232,6 +258,8 @@ group_norm_kernel(TO *__restrict__ y, float *x, const int32_t *__restrict__ rows
         }
         part += double(v * v);
       }
+    }
+    if (active) {
       part = wave_sum(part);
       if (lane == 0) wave_part[wave] = part;
     }
@@ -241,11 +269,24 @@ group_norm_kernel(TO *__restrict__ y, float *x, const int32_t *__restrict__ rows
       double total = 0.0;
       for (int j = 0; j < wpg; ++j) total += wave_part[(wave / wpg) * wpg + j];
       const float inv = 1.0f / sqrtf(float(total / double(gw)) + eps);
-      for (int i = lane + 64 * k; i < gw; i += 64 * wpg) {
-        const size_t e = size_t(g) * gw + i;
-        float o = xr[e] * inv;
-        if (w) o = o * ld_dyn(w, w_dtype, e);
-        st_f(yr, e, o);
+      if (vec) {
+        for (int i = 4 * (lane + 64 * k); i < gw; i += 256 * wpg) {
+          const size_t e = size_t(g) * gw + i;
+          const float4 v = *reinterpret_cast<const float4 *>(xr + e);
+          float o4[4] = {v.x * inv, v.y * inv, v.z * inv, v.w * inv};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (w) o4[j] = o4[j] * ld_dyn(w, w_dtype, e + j);
+            st_f(yr, e + j, o4[j]);
+          }
+        }
+      } else {
+        for (int i = lane + 64 * k; i < gw; i += 64 * wpg) {
+          const size_t e = size_t(g) * gw + i;
+          float o = xr[e] * inv;
+          if (w) o = o * ld_dyn(w, w_dtype, e);
+          st_f(yr, e, o);
+        }
       }
     }
     __syncthreads();

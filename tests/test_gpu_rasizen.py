@@ -269,6 +269,54 @@ def test_greedy_generation_through_the_entry_point(folders):
                 assert row[t] >= row.max() - 2 * BF16_WORST * row.std(), (name, i)
 
 
+def test_command_line_and_trace_replay(folders, tmp_path):
+    """The command line generates from a folder and from a configuration file of this design; the
+    replay program feeds a prompt, then its next tokens one by one beside a second request, frees
+    one and goes on, and writes the logits the plain implementation gives."""
+    import subprocess
+    import sys
+    from conftest import ROOT
+    name = "M"
+    ps = prompts(name, [4, 10], seed=9)
+    tokens = tmp_path / "prompts.txt"
+    tokens.write_text("\n".join(" ".join(map(str, p)) for p in ps) + "\n")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "-m", folders[name], "--tokens", str(tokens), "-n", "6",
+           "--dtype", "fp32", "--stop", ""]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    got = [[int(t) for t in line.split()] for line in out.stdout.strip().splitlines()]
+    assert got == [R.greedy(CONFIGS[name], _PLAIN[name], p, 6) for p in ps]
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(CONFIGS["L"]))
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "--random", str(cfg_file), "--seed", "3",
+           "--tokens", str(tokens), "-n", "5", "--temperature", "0.8", "--sample-seed", "11", "--top-k", "20"]
+    one = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    two = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert one.returncode == 0 and one.stdout == two.stdout and len(one.stdout.split()) == 10, one.stderr
+    # replay
+    a, b = prompts(name, [75, 12], seed=10)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:70], "want": [0, 69]}, {"id": "b", "tokens": b[:9], "want": [8]}], "end": []}]
+    for k in range(3):
+        steps.append({"step": k + 1, "entries": [{"id": "a", "tokens": [a[70 + k]], "want": [0]},
+                                                 {"id": "b", "tokens": [b[9 + k]], "want": [] if k == 1 else [0]}],
+                      "end": ["b"] if k == 2 else []})
+    steps.append({"step": 4, "entries": [{"id": "a", "tokens": a[73:75], "want": [1]}], "end": ["a"]})
+    outdir = tmp_path / "out"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name], "--dtype", "float32",
+                          "--out", str(outdir), "--max-tokens", "256"], input="\n".join(json.dumps(x) for x in steps) + "\n",
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert [ln for ln in run.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(5)]
+    wa, wb = want_logits(name, a), want_logits(name, b)
+    vocab = CONFIGS[name]["vocab"]
+    read = lambda i: np.fromfile(outdir / f"{i}.f32", dtype="<f4").reshape(-1, vocab)
+    close(read(0), np.stack([wa[0], wa[69], wb[8]]), "float32", "replay, prompts")
+    close(read(1), np.stack([wa[70], wb[9]]), "float32", "replay, first single tokens")
+    close(read(2), wa[71:72], "float32", "replay, a step where one request wants nothing")
+    close(read(3), np.stack([wa[72], wb[11]]), "float32", "replay, last step of the short request")
+    close(read(4), wa[74:75], "float32", "replay, two more tokens alone")
+
+
 # ---- mechanisms alone ---------------------------------------------------------------------------
 def runtime(dtype):
     from sonicboom_amd.parts import Runtime
