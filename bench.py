@@ -739,6 +739,8 @@ def design_roofline(label, us, calls, rows, depth, batch, width, cfgs):
     nbytes = flops = None
     if label.startswith("gemm"):
         n, k = (int(v) for v in label.split()[-1].split("x"))
+        if n == cfgs["vocab"] and not decode:
+            rows = 1                     # the head runs on the wanted rows only: the prompt's last
         nbytes, flops = 2 * n * k + 2 * rows * k + 4 * rows * (n // (2 if "gated" in label else 1)), 2 * rows * n * k
     elif label.startswith("rmsnorm") or label == "reduce_resid_norm":
         nbytes = rows * width * (4 + 2 + (8 if label == "reduce_resid_norm" else 0))
@@ -780,7 +782,8 @@ def design_comparison(a) -> int:
             model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
             heads = width // 128
             cfgs = {"heads": heads, "rank": 512, "rot": 64, "window": 4096 if design == "rasizen" else 1 << 30,
-                    "gru": 2 * width, "ff": 4 * width, "kvw": max(1, heads // 4) * 128}
+                    "gru": 2 * width, "ff": 4 * width, "kvw": max(1, heads // 4) * 128,
+                    "vocab": cfg.get("vocab", cfg.get("vocab_size"))}
             eng = Engine(model, (a.prompt + a.steps + a.warmup + 128) * (a.batch + 1), max_positions=0)
             prompt = [int(t) for t in rng.integers(0, cfg.get("vocab", cfg.get("vocab_size")), size=a.prompt)]
 

@@ -321,24 +321,46 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
 }
 
 // out[column, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M), M the largest m_s: the shares of
-// a column's keys that n_splits blocks worked on, put together.  A block a column.
+// a column's keys that n_splits blocks worked on, put together.  A block a column; the shares'
+// weights 2^(m_s - M) wait in LDS, and a thread asks for eight shares of its numbers at a time.
+constexpr int kMaxSplits = 512;
+
 __global__ void __launch_bounds__(256)
 latent_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
                     int n_splits, size_t n_columns, int rank) {
+  __shared__ float weight[kMaxSplits];
+  __shared__ float wave_l[4];
   const size_t column = blockIdx.x;
+  const int tid = threadIdx.x;
   float m = -__builtin_inff();
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part_ml[2 * (size_t(s) * n_columns + column)]);
+  for (int s = tid; s < n_splits; s += 256) m = fmaxf(m, part_ml[2 * (size_t(s) * n_columns + column)]);
+  m = wave_max(m);
+  if ((tid & 63) == 0) wave_l[tid >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(wave_l[0], wave_l[1]), fmaxf(wave_l[2], wave_l[3]));
+  __syncthreads();
   float l = 0.0f;
-  for (int s = 0; s < n_splits; ++s) {
+  for (int s = tid; s < n_splits; s += 256) {
     const float ms = part_ml[2 * (size_t(s) * n_columns + column)];
-    if (ms > -__builtin_inff()) l += part_ml[2 * (size_t(s) * n_columns + column) + 1] * exp2f(ms - m);
+    const float ws = ms > -__builtin_inff() ? exp2f(ms - m) : 0.0f;
+    weight[s] = ws;
+    l += part_ml[2 * (size_t(s) * n_columns + column) + 1] * ws;
   }
+  l = wave_sum(l);
+  if ((tid & 63) == 0) wave_l[tid >> 6] = l;
+  __syncthreads();
+  l = (wave_l[0] + wave_l[1]) + (wave_l[2] + wave_l[3]);
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-  for (int d = threadIdx.x; d < rank; d += 256) {
+  for (int d = tid; d < rank; d += 256) {
     float acc = 0.0f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = part_ml[2 * (size_t(s) * n_columns + column)];
-      if (ms > -__builtin_inff()) acc += part_o[(size_t(s) * n_columns + column) * rank + d] * exp2f(ms - m);
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = part_o[(size_t(min(s0 + u, n_splits - 1)) * n_columns + column) * rank + d];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < n_splits) acc += v[u] * weight[s0 + u];
     }
     out[column * rank + d] = f32_to_bf16(acc * inv);
   }
@@ -428,7 +450,7 @@ extern "C" int sb_latent_attention_bf16(void *out, const void *q, const void *ca
   SB_REQUIRE(n_tiles >= 0 && heads > 0 && max_pages > 0 && n_pages_total > 0 && window >= 0,
              "sb_latent_attention_bf16: bad sizes");
   SB_REQUIRE(tile_rows == 16 || tile_rows == 1, "sb_latent_attention_bf16: tiles of 16 rows or of one");
-  SB_REQUIRE(n_splits >= 1 && n_splits <= 65535 && n_rows >= 0 && (n_splits == 1 || (part_o && part_ml)),
+  SB_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && n_rows >= 0 && (n_splits == 1 || (part_o && part_ml)),
              "sb_latent_attention_bf16: shares of the keys need their scratch");
   SB_SUPPORT(sb_latent_attention_bf16_ok(rank, rot_dim), "sb_latent_attention_bf16: a latent row of %d + %d is not taken",
              rank, rot_dim);

@@ -226,11 +226,15 @@ group_norm_kernel(TO *__restrict__ y, float *x, const int32_t *__restrict__ rows
         const size_t e = size_t(g) * gw + i;
         float4 v;
         if (pr) {
-          float4 acc = *reinterpret_cast<const float4 *>(pr + e);
-          for (int s = 1; s < n_slices; ++s) {
-            const float4 p4 = *reinterpret_cast<const float4 *>(pr + size_t(s) * slice_stride + e);
-            acc.x += p4.x; acc.y += p4.y; acc.z += p4.z; acc.w += p4.w;
-          }
+          // every slice's load goes out before the first sum (a slice past the last is the last again, unused)
+          float4 p4[kMaxSlices];
+#pragma unroll
+          for (int s = 0; s < kMaxSlices; ++s)
+            p4[s] = *reinterpret_cast<const float4 *>(pr + size_t(min(s, n_slices - 1)) * slice_stride + e);
+          float4 acc = p4[0];
+#pragma unroll
+          for (int s = 1; s < kMaxSlices; ++s)
+            if (s < n_slices) { acc.x += p4[s].x; acc.y += p4[s].y; acc.z += p4[s].z; acc.w += p4[s].w; }
           if (bias) {
             acc.x += ld_dyn(bias, bias_dtype, e); acc.y += ld_dyn(bias, bias_dtype, e + 1);
             acc.z += ld_dyn(bias, bias_dtype, e + 2); acc.w += ld_dyn(bias, bias_dtype, e + 3);
@@ -322,6 +326,7 @@ extern "C" int sb_reduce_scaled_group_norm(void *y, int y_dtype, float *x, const
                                            int n_rows, int width, int groups, float eps, int do_norm, void *stream) {
   SB_REQUIRE(x && partial && (!do_norm || y), "sb_reduce_scaled_group_norm: null pointer");
   SB_REQUIRE(n_rows >= 0 && width > 0 && n_slices >= 1 && groups > 0, "sb_reduce_scaled_group_norm: bad sizes");
+  SB_SUPPORT(n_slices <= kMaxSlices, "sb_reduce_scaled_group_norm: %d slices, at most %d", n_slices, kMaxSlices);
   SB_REQUIRE(width % groups == 0, "sb_reduce_scaled_group_norm: %d groups do not divide a row of %d", groups, width);
   SB_REQUIRE((!do_norm || sb::valid_dtype(y_dtype)) && (!bias || sb::valid_dtype(bias_dtype)) &&
                  (!w || sb::valid_dtype(w_dtype)),

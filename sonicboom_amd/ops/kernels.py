@@ -981,7 +981,7 @@ def latent_attention_mfma_ok(q_dtype, cache_dtype, rank: int, rot_dim: int) -> b
 
 
 LATENT_SPLIT_BLOCKS = 512       # blocks a step of few rows aims at by sharing out its keys
-LATENT_SPLIT_KEYS = 64          # keys a share has at least
+LATENT_SPLIT_KEYS = 128         # keys a share has at least (64: 45 us, 128: 41, 256: 50 for 8 rows over 2,049 keys of 576 numbers)
 
 
 def latent_attention_mfma(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Tensor, row_pos: torch.Tensor,
