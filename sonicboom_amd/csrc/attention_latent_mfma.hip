@@ -65,18 +65,27 @@ head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstri
       for (int j = 0; j < 4; ++j) acc[j] = mfma16(as_bf16x8(av[u][j]), as_bf16x8(b[u]), acc[j]);
   }
   if (t >= n_rows) return;
+  // a lane holds four neighbouring outputs of its row: one 8-byte store where the row's layout allows
+  const bool wide = (out_stride % 4 == 0) && (out_hstride % 4 == 0) && (reinterpret_cast<uintptr_t>(out) % 8 == 0);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
+    const int ob = o0 + 16 * j + 4 * g;
+    float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int o = o0 + 16 * j + 4 * g + i;
-      if (o >= n_out) continue;
-      float v = acc[j][i];
-      if (GATED) {
-        const float gv = gate[size_t(t) * gate_stride + size_t(a) * n_out + o];
-        v = v * (1.0f / (1.0f + expf(-gv)));
+      v[i] = acc[j][i];
+      if (GATED && ob + i < n_out) {
+        const float gv = gate[size_t(t) * gate_stride + size_t(a) * n_out + ob + i];
+        v[i] = v[i] * (1.0f / (1.0f + expf(-gv)));
       }
-      out[size_t(t) * out_stride + size_t(a) * out_hstride + o] = f32_to_bf16(v);
+    }
+    bf16_t *dst = out + size_t(t) * out_stride + size_t(a) * out_hstride + ob;
+    if (wide && ob + 3 < n_out) {
+      *reinterpret_cast<uint2 *>(dst) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (ob + i < n_out) dst[i] = f32_to_bf16(v[i]);
     }
   }
 }

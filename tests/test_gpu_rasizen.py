@@ -129,7 +129,7 @@ def prompts(name, lengths, seed=0):
 # bfloat16 is measured in spreads of the logits (their standard deviation): the largest difference
 # and the root mean square of all differences of a request.
 F32_BOUND = 2e-4
-BF16_WORST, BF16_RMS = 0.25, 0.05
+BF16_WORST, BF16_RMS = 0.28, 0.019      # what the whole file measured (0.2007 and 0.0135: the models are sharpened) times 1.4
 helpers.BF16_MAX["recurrent and latent"], helpers.BF16_RMS["recurrent and latent"] = BF16_WORST, BF16_RMS
 
 
