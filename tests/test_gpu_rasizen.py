@@ -315,6 +315,19 @@ def test_command_line_and_trace_replay(folders, tmp_path):
     close(read(2), wa[71:72], "float32", "replay, a step where one request wants nothing")
     close(read(3), np.stack([wa[72], wb[11]]), "float32", "replay, last step of the short request")
     close(read(4), wa[74:75], "float32", "replay, two more tokens alone")
+    # many short requests at once, with no more --max-tokens than the tokens they hold: every one of them
+    # takes a page of its own in the cache, which the program makes room for
+    shorts = prompts(name, [3] * 14, seed=12)
+    steps = [{"step": 0, "entries": [{"id": f"s{i}", "tokens": p[:2], "want": [1]} for i, p in enumerate(shorts)], "end": []},
+             {"step": 1, "entries": [{"id": f"s{i}", "tokens": p[2:], "want": [0]} for i, p in enumerate(shorts)],
+              "end": [f"s{i}" for i in range(14)]}]
+    outdir2 = tmp_path / "out2"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name], "--dtype", "bfloat16",
+                          "--out", str(outdir2), "--max-tokens", str(3 * 14)], input="\n".join(json.dumps(x) for x in steps) + "\n",
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    got = np.fromfile(outdir2 / "1.f32", dtype="<f4").reshape(-1, vocab)
+    close(got, np.stack([want_logits(name, p)[2] for p in shorts]), "bfloat16", "replay, fourteen short requests")
 
 
 # ---- mechanisms alone ---------------------------------------------------------------------------
