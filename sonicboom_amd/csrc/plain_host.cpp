@@ -220,6 +220,181 @@ int sbp_attention(float *out, const float *q, int q_stride, const float *k_cache
   return 0;
 }
 
+// ---- the gated recurrence and latent attention ---------------------------------------------------
+// The norm taken over each of `groups` equal consecutive parts of the row; the weight spans the row.
+int sbp_rmsnorm_grouped(float *y, const float *x, const float *w, const int32_t *rows, int n_rows, int width,
+                        int groups, float eps) {
+  if (!y || !x || n_rows < 0 || width <= 0 || groups <= 0 || width % groups || eps < 0.f) return 1;
+  const int gw = width / groups;
+  for (int r = 0; r < n_rows; ++r) {
+    const float *xr = x + size_t(rows ? rows[r] : r) * width;
+    for (int g = 0; g < groups; ++g) {
+      double sum = 0.0;
+      for (int i = 0; i < gw; ++i) sum += double(xr[g * gw + i] * xr[g * gw + i]);
+      const float inv = 1.0f / std::sqrt(float(sum / double(gw)) + eps);
+      for (int i = g * gw; i < (g + 1) * gw; ++i) {
+        float o = xr[i] * inv;
+        if (w) o = o * w[i];
+        y[size_t(r) * width + i] = o;
+      }
+    }
+  }
+  return 0;
+}
+
+// x[t,:] += scale * (sum of the slices in ascending order (+ bias)); with do_norm y = the grouped norm of x.
+int sbp_reduce_scaled_group_norm(float *y, float *x, const float *partial, int n_slices, const float *bias,
+                                 float scale, const float *w, int n_rows, int width, int groups, float eps,
+                                 int do_norm) {
+  if (!x || !partial || (do_norm && !y) || n_rows < 0 || width <= 0 || n_slices < 1 || groups <= 0 || width % groups)
+    return 1;
+  for (int t = 0; t < n_rows; ++t)
+    for (int i = 0; i < width; ++i) {
+      float acc = partial[size_t(t) * width + i];
+      for (int s = 1; s < n_slices; ++s) acc += partial[(size_t(s) * n_rows + t) * width + i];
+      if (bias) acc += bias[i];
+      x[size_t(t) * width + i] = std::fma(acc, scale, x[size_t(t) * width + i]);
+    }
+  return do_norm ? sbp_rmsnorm_grouped(y, x, w, nullptr, n_rows, width, groups, eps) : 0;
+}
+
+int sbp_add_scaled(float *resid, const float *y, float scale, size_t n) {
+  if (!resid || !y) return 1;
+  for (size_t i = 0; i < n; ++i) resid[i] = std::fma(y[i], scale, resid[i]);
+  return 0;
+}
+
+// kind 1: SiLU, 2: the tanh form of GELU, 3: xIELU with params (p, q): softplus(p) z^2 + z/2 for z > 0,
+// (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 else.
+int sbp_activate(float *out, const float *in, size_t n, int kind, const float *params) {
+  if (!out || !in || kind < 1 || kind > 3 || (kind == 3 && !params)) return 1;
+  auto softplus = [](float a) { return a > 20.0f ? a : std::log1p(std::exp(a)); };
+  const float ap = kind == 3 ? softplus(params[0]) : 0.f, an = kind == 3 ? 0.5f + softplus(params[1]) : 0.f;
+  for (size_t i = 0; i < n; ++i) {
+    const float z = in[i];
+    if (kind == 3) out[i] = z > 0.0f ? ap * z * z + 0.5f * z : an * (std::expm1(z) - z) + 0.5f * z;
+    else if (kind == 2) out[i] = 0.5f * z * (1.0f + std::tanh(0.79788456080286535588f * z * (1.0f + 0.044715f * z * z)));
+    else out[i] = z / (1.0f + std::exp(-z));
+  }
+  return 0;
+}
+
+// minGRU over the rows of every sequence in order: p [rows, 3 width] = (a | u | g) before their activations.
+int sbp_mingru_scan(float *out, const float *p, float *state, const int32_t *cu_rows, const int32_t *slots,
+                    int n_seqs, int width) {
+  if (!out || !p || !state || !cu_rows || !slots || n_seqs < 0 || width <= 0) return 1;
+  auto sigmoid = [](float a) { return 1.0f / (1.0f + std::exp(-a)); };
+  for (int s = 0; s < n_seqs; ++s)
+    for (int ch = 0; ch < width; ++ch) {
+      float st = state[size_t(slots[s]) * width + ch];
+      for (int r = cu_rows[s]; r < cu_rows[s + 1]; ++r) {
+        const float *row = p + size_t(r) * 3 * width;
+        const float z = sigmoid(row[ch]), u = row[width + ch], g = row[2 * width + ch];
+        const float cand = u >= 0.0f ? u + 0.5f : sigmoid(u);
+        st = (1.0f - z) * st + z * cand;
+        out[size_t(r) * width + ch] = st * (g * sigmoid(g));
+      }
+      state[size_t(slots[s]) * width + ch] = st;
+    }
+  return 0;
+}
+
+int sbp_latent_prepare(float *q_plain, float *q_latent, const float *p, int row_stride, int q_off, int kv_off,
+                       const float *c_weight, float eps, const float *inv_freq, int rot_dims, int interleaved,
+                       const int32_t *row_pos, const int32_t *row_seq, float *cache, const int32_t *page_table,
+                       int max_pages, int n_pages_total, int n_rows, int heads, int dim, int rot_dim, int rank) {
+  if (!q_plain || !q_latent || !p || !row_pos || !row_seq || rot_dims % 2 || rot_dims > rot_dim) return 1;
+  if (kv_off >= 0 && (!cache || !page_table)) return 1;
+  const int latent = rank + rot_dim, hd = dim + rot_dim;
+  auto turn = [&](const float *src, float *dst, float pos) {      // the rotated part of a key or of a query head
+    for (int j = 0; j < rot_dims / 2; ++j) {
+      const int i0 = interleaved ? 2 * j : j, i1 = interleaved ? 2 * j + 1 : j + rot_dims / 2;
+      const float a = pos * inv_freq[j], c = std::cos(a), s = std::sin(a);
+      const float x0 = src[i0], x1 = src[i1];
+      dst[i0] = x0 * c - x1 * s;
+      dst[i1] = x0 * s + x1 * c;
+    }
+    for (int i = rot_dims; i < rot_dim; ++i) dst[i] = src[i];
+  };
+  for (int t = 0; t < n_rows; ++t) {
+    const float *pr = p + size_t(t) * row_stride;
+    const int pos = row_pos[t];
+    if (kv_off >= 0) {
+      const int lp = pos / kPage;
+      const int page = lp < max_pages ? page_table[size_t(row_seq[t]) * max_pages + lp] : -1;
+      if (page >= 0 && page < n_pages_total) {
+        float *dst = cache + (size_t(page) * kPage + pos % kPage) * latent;
+        double sum = 0.0;
+        for (int i = 0; i < rank; ++i) sum += double(pr[kv_off + i] * pr[kv_off + i]);
+        const float inv = 1.0f / std::sqrt(float(sum / double(rank)) + eps);
+        for (int i = 0; i < rank; ++i) {
+          float o = pr[kv_off + i] * inv;
+          if (c_weight) o = o * c_weight[i];
+          dst[i] = o;
+        }
+        turn(pr + kv_off + rank, dst + rank, float(pos));
+      }
+    }
+    for (int a = 0; a < heads; ++a) {
+      for (int d = 0; d < dim; ++d) q_plain[(size_t(t) * heads + a) * dim + d] = pr[q_off + a * hd + d];
+      turn(pr + q_off + a * hd + dim, q_latent + (size_t(t) * heads + a) * latent + rank, float(pos));
+    }
+  }
+  return 0;
+}
+
+// out[t, a, o] = sum_i W[a][o][i] in[t, a, i] in ascending i (times sigmoid(gate[t, a n_out + o])).
+int sbp_head_product(float *out, int out_stride, int out_hstride, const float *in, int in_stride, int in_hstride,
+                     const float *w, const float *gate, int gate_stride, int n_rows, int heads, int n_in, int n_out) {
+  if (!out || !in || !w || n_rows < 0 || heads <= 0 || n_in <= 0 || n_out <= 0) return 1;
+  for (int t = 0; t < n_rows; ++t)
+    for (int a = 0; a < heads; ++a)
+      for (int o = 0; o < n_out; ++o) {
+        float acc = 0.0f;
+        for (int i = 0; i < n_in; ++i)
+          acc = std::fma(in[size_t(t) * in_stride + size_t(a) * in_hstride + i], w[(size_t(a) * n_out + o) * n_in + i], acc);
+        if (gate) acc = acc * (1.0f / (1.0f + std::exp(-gate[size_t(t) * gate_stride + size_t(a) * n_out + o])));
+        out[size_t(t) * out_stride + size_t(a) * out_hstride + o] = acc;
+      }
+  return 0;
+}
+
+// Softmax attention of every (row, head) over the cached latent rows it sees; the result is the
+// weighted sum of the rows' first rank numbers.  Two passes over the keys, in double.
+int sbp_latent_attention(float *out, const float *q, const float *cache, const int32_t *page_table, int max_pages,
+                         int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads,
+                         int rank, int rot_dim, float scale, int window) {
+  if (!out || !q || !cache || !page_table || !row_pos || !row_seq || rank <= 0 || rot_dim < 0) return 1;
+  const int latent = rank + rot_dim;
+  for (int t = 0; t < n_rows; ++t) {
+    const int pos = row_pos[t], lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+    for (int a = 0; a < heads; ++a) {
+      const float *qr = q + (size_t(t) * heads + a) * latent;
+      std::vector<double> s;
+      std::vector<const float *> rows;
+      for (int j = lo; j <= pos; ++j) {
+        const int page = j / kPage < max_pages ? page_table[size_t(row_seq[t]) * max_pages + j / kPage] : -1;
+        if (page < 0 || page >= n_pages_total) continue;
+        const float *kr = cache + (size_t(page) * kPage + j % kPage) * latent;
+        double dot = 0.0;
+        for (int d = 0; d < latent; ++d) dot += double(qr[d]) * double(kr[d]);
+        s.push_back(dot * double(scale));
+        rows.push_back(kr);
+      }
+      std::vector<double> acc(rank, 0.0);
+      double m = -std::numeric_limits<double>::infinity(), l = 0.0;
+      for (double v : s) m = std::max(m, v);
+      for (size_t k = 0; k < s.size(); ++k) {
+        const double pk = std::exp(s[k] - m);
+        l += pk;
+        for (int d = 0; d < rank; ++d) acc[d] += pk * double(rows[k][d]);
+      }
+      for (int d = 0; d < rank; ++d) out[(size_t(t) * heads + a) * rank + d] = l > 0.0 ? float(acc[d] / l) : 0.0f;
+    }
+  }
+  return 0;
+}
+
 // ids[r] = index of the first maximum of logits[r,:].
 int sbp_argmax(int32_t *ids, const float *logits, int n_rows, int vocab) {
   if (!ids || !logits || n_rows < 0 || vocab <= 0) return 1;

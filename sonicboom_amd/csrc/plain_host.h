@@ -29,6 +29,26 @@ int sbp_attention(float *out, const float *q, int q_stride, const float *k_cache
                   const int32_t *page_table, int max_pages, int n_pages_total, const int32_t *row_pos,
                   const int32_t *row_seq, int n_rows, int heads_q, int heads_kv, int head_dim, float scale,
                   int window);
+/* The kernels of the gated recurrence and of latent attention (csrc/recurrent.hip, csrc/attention_latent.hip),
+ * the grouped norm, the scaled add and the activations. */
+int sbp_rmsnorm_grouped(float *y, const float *x, const float *w, const int32_t *rows, int n_rows, int width,
+                        int groups, float eps);
+int sbp_reduce_scaled_group_norm(float *y, float *x, const float *partial, int n_slices, const float *bias,
+                                 float scale, const float *w, int n_rows, int width, int groups, float eps,
+                                 int do_norm);
+int sbp_add_scaled(float *resid, const float *y, float scale, size_t n);
+int sbp_activate(float *out, const float *in, size_t n, int kind, const float *params);   /* kind: an sb_act */
+int sbp_mingru_scan(float *out, const float *p, float *state, const int32_t *cu_rows, const int32_t *slots,
+                    int n_seqs, int width);
+int sbp_latent_prepare(float *q_plain, float *q_latent, const float *p, int row_stride, int q_off, int kv_off,
+                       const float *c_weight, float eps, const float *inv_freq, int rot_dims, int interleaved,
+                       const int32_t *row_pos, const int32_t *row_seq, float *cache, const int32_t *page_table,
+                       int max_pages, int n_pages_total, int n_rows, int heads, int dim, int rot_dim, int rank);
+int sbp_head_product(float *out, int out_stride, int out_hstride, const float *in, int in_stride, int in_hstride,
+                     const float *w, const float *gate, int gate_stride, int n_rows, int heads, int n_in, int n_out);
+int sbp_latent_attention(float *out, const float *q, const float *cache, const int32_t *page_table, int max_pages,
+                         int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads,
+                         int rank, int rot_dim, float scale, int window);
 int sbp_argmax(int32_t *ids, const float *logits, int n_rows, int vocab);
 int sbp_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
                  const int32_t *item_count, int n_items, float repeat_penalty, float presence_penalty,

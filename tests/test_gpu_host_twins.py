@@ -309,3 +309,153 @@ def test_kernels_equal_their_host_twins():
                        float(np.log(np.float32(min_p))) if min_p > 0.0 else None,
                        float(np.float32(top_p)) if 0.0 < top_p < 1.0 else None, seed)
         assert got.cpu().numpy().tolist() == want.tolist(), case
+
+
+# ---- the gated recurrence and latent attention: twins against NumPy, kernels against twins -----------
+from plain import rasizen_plain as RP  # noqa: E402
+
+CF = ctypes.c_float
+
+
+def latent_twin_setup(n=150, heads=3, dim=8, rot_dim=8, dims=6, rank=16, width=40, seed=3):
+    """Rows of a latent-attention layer's input product, its weights, and a page table that scatters
+    one sequence's pages."""
+    rng = np.random.default_rng(seed)
+    stride = heads * (dim + rot_dim) + 5 + rank + rot_dim                # five numbers between queries and the latent's part
+    p = rng.standard_normal((n, stride)).astype(np.float32)
+    cw = (1.0 + 0.1 * rng.standard_normal(rank)).astype(np.float32)
+    inv_freq = (100.0 ** (-2.0 * np.arange(dims // 2) / dims)).astype(np.float32)
+    pages = (n + 63) // 64
+    table = i32([[5, 2, 7][:pages]])
+    pos, seq = i32(np.arange(n)), i32(np.zeros(n))
+    return p, cw, inv_freq, table, pos, seq, stride, heads * (dim + rot_dim) + 5
+
+
+def host_latent(lib, p, cw, inv_freq, table, pos, seq, stride, kv_off, heads, dim, rot_dim, dims, rank, scale, window, uk):
+    n, latent = p.shape[0], rank + rot_dim
+    cache = np.zeros((8, 64, latent), np.float32)
+    qp, ql = np.zeros((n, heads, dim), np.float32), np.zeros((n, heads, latent), np.float32)
+    assert lib.sbp_latent_prepare(ptr(qp), ptr(ql), ptr(p), C(stride), C(0), C(kv_off), ptr(cw), CF(1e-5), ptr(inv_freq),
+                                  C(dims), C(1), ptr(pos), ptr(seq), ptr(cache), ptr(table), C(table.shape[1]), C(8), C(n),
+                                  C(heads), C(dim), C(rot_dim), C(rank)) == 0
+    assert lib.sbp_head_product(ptr(ql), C(heads * latent), C(latent), ptr(qp), C(heads * dim), C(dim), ptr(uk), None, C(0),
+                                C(n), C(heads), C(dim), C(rank)) == 0
+    out = np.zeros((n, heads, rank), np.float32)
+    assert lib.sbp_latent_attention(ptr(out), ptr(ql), ptr(cache), ptr(table), C(table.shape[1]), C(8), ptr(pos), ptr(seq),
+                                    C(n), C(heads), C(rank), C(rot_dim), CF(scale), C(window)) == 0
+    return qp, ql, cache, out
+
+
+def test_recurrent_and_latent_twins_agree_with_the_plain_implementation():
+    lib = twins()
+    for name in ("sbp_rmsnorm_grouped", "sbp_reduce_scaled_group_norm", "sbp_add_scaled", "sbp_activate", "sbp_mingru_scan",
+                 "sbp_latent_prepare", "sbp_head_product", "sbp_latent_attention"):
+        getattr(lib, name).restype = ctypes.c_int
+    # grouped norm; slices, multiplier, residual and grouped norm
+    x, w = f32(5, 60, seed=1, scale=3.0), f32(60, seed=2)
+    y = np.empty_like(x)
+    assert lib.sbp_rmsnorm_grouped(ptr(y), ptr(x), ptr(w), None, C(5), C(60), C(3), CF(1e-4)) == 0
+    assert np.allclose(y, RP.grouped_rms_norm(x, w, 1e-4, 3), atol=1e-5)
+    part, b = f32(2, 5, 60, seed=3), f32(60, seed=4)
+    x2, y2 = x.copy(), np.empty_like(x)
+    assert lib.sbp_reduce_scaled_group_norm(ptr(y2), ptr(x2), ptr(part), C(2), ptr(b), CF(0.3), ptr(w), C(5), C(60), C(3),
+                                            CF(1e-4), C(1)) == 0
+    want = x + 0.3 * (part[0] + part[1] + b)
+    assert np.allclose(x2, want, atol=1e-5) and np.allclose(y2, RP.grouped_rms_norm(want, w, 1e-4, 3), atol=1e-5)
+    # activation
+    z, pq = np.linspace(-8, 8, 101).astype(np.float32), np.asarray([0.4, -0.3], np.float32)
+    out = np.empty_like(z)
+    assert lib.sbp_activate(ptr(out), ptr(z), ctypes.c_size_t(101), C(3), ptr(pq)) == 0
+    assert np.allclose(out, RP.xielu(z, 0.4, -0.3), atol=1e-5, rtol=1e-5)
+    # recurrence: two sequences of 7 and 30 rows, the second from a state that is not zero
+    width = 12
+    p, state = f32(37, 3 * width, seed=5, scale=2.0), np.zeros((4, width), np.float32)
+    state[3] = f32(width, seed=6)
+    start = state[3].copy()
+    out = np.empty((37, width), np.float32)
+    assert lib.sbp_mingru_scan(ptr(out), ptr(p), ptr(state), ptr(i32([0, 7, 37])), ptr(i32([1, 3])), C(2), C(width)) == 0
+    for rows, s0, slot in ((slice(0, 7), None, 1), (slice(7, 37), start, 3)):
+        zz, u, g = RP.sigmoid(p[rows, :width]), p[rows, width:2 * width], p[rows, 2 * width:]
+        s = RP.mingru_scan(zz, np.where(u >= 0, u + 0.5, RP.sigmoid(u)), start=s0)
+        assert np.allclose(out[rows], s * g * RP.sigmoid(g), atol=1e-5) and np.allclose(state[slot], s[-1], atol=1e-5)
+    # latent attention: prepare, carry the queries over, attend
+    heads, dim, rot_dim, dims, rank, scale, window = 3, 8, 8, 6, 16, 0.3, 70
+    p, cw, inv_freq, table, pos, seq, stride, kv_off = latent_twin_setup()
+    uk = f32(heads, rank, dim, seed=7, scale=0.4)            # [head, out, in]: W_uk,a^T
+    qp, ql, cache, out = host_latent(lib, p, cw, inv_freq, table, pos, seq, stride, kv_off, heads, dim, rot_dim, dims, rank,
+                                     scale, window, uk)
+    mx = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": 1, "kv_rank": rank, "scale": scale,
+          "rot": {"base": 100.0, "dims": dims}, "mask": {"size": window}}
+    n = p.shape[0]
+    c = RP.grouped_rms_norm(p[:, kv_off:kv_off + rank], cw, 1e-5, 1)
+    r = RP.rotate_pairs(p[:, kv_off + rank:kv_off + rank + rot_dim], pos, dims, 100.0)
+    rows = np.concatenate([c, r], -1)
+    stored = cache[table[0][np.arange(n) // 64], np.arange(n) % 64]
+    assert np.allclose(stored, rows, atol=2e-5)
+    q = p[:, :heads * (dim + rot_dim)].reshape(n, heads, dim + rot_dim).astype(np.float64)
+    keys = np.concatenate([np.einsum("ard,tr->tad", uk.astype(np.float64), c), np.repeat(r[:, None], heads, 1)], -1)
+    qq = np.concatenate([q[..., :dim], RP.rotate_pairs(q[..., dim:], pos, dims, 100.0)], -1)
+    want = RP.windowed_softmax_attention(qq, keys, np.repeat(c[:, None], heads, 1), scale, window)
+    assert np.allclose(out, want, atol=3e-5)
+
+
+@pytest.mark.gpu
+def test_recurrent_and_latent_kernels_equal_their_host_twins():
+    from sonicboom_amd import ops
+    lib = twins()
+    for name in ("sbp_rmsnorm_grouped", "sbp_reduce_scaled_group_norm", "sbp_add_scaled", "sbp_activate", "sbp_mingru_scan",
+                 "sbp_latent_prepare", "sbp_head_product", "sbp_latent_attention"):
+        getattr(lib, name).restype = ctypes.c_int
+    dev = lambda a: None if a is None else torch.from_numpy(a).to(DEV)  # noqa: E731
+    for width, groups, n_rows in ((96, 2, 3), (520, 4, 70), (66, 6, 5), (4096, 1, 2)):
+        x, w = f32(n_rows, width, seed=width, scale=2.0), f32(width, seed=2)
+        want = np.empty_like(x)
+        assert lib.sbp_rmsnorm_grouped(ptr(want), ptr(x), ptr(w), None, C(n_rows), C(width), C(groups), CF(1e-6)) == 0
+        assert np.allclose(ops.rmsnorm(dev(x), dev(w), 1e-6, F32, groups=groups).cpu().numpy() if groups > 1 else
+                           ops.rmsnorm(dev(x), dev(w), 1e-6, F32).cpu().numpy(), want, atol=1e-6, rtol=1e-6)
+        part, b = f32(3, n_rows, width, seed=7), f32(width, seed=8)
+        x_host, y_host = x.copy(), np.empty_like(x)
+        assert lib.sbp_reduce_scaled_group_norm(ptr(y_host), ptr(x_host), ptr(part), C(3), ptr(b), CF(0.35), ptr(w), C(n_rows),
+                                                C(width), C(groups), CF(1e-5), C(1)) == 0
+        x_dev = dev(x)
+        y_dev = ops.reduce_resid_norm(dev(part), dev(b), x_dev, dev(w), 1e-5, F32, scale=0.35, groups=groups)
+        assert np.allclose(x_dev.cpu().numpy(), x_host, atol=1e-6, rtol=1e-6) and np.allclose(y_dev.cpu().numpy(), y_host, atol=2e-6, rtol=2e-6)
+    # scaled add, activation
+    r, y = f32(1000, seed=1), f32(1000, seed=2)
+    r_host, r_dev = r.copy(), dev(r)
+    lib.sbp_add_scaled(ptr(r_host), ptr(y), CF(0.3), ctypes.c_size_t(1000))
+    ops.add_scaled(r_dev, dev(y), 0.3)
+    assert np.allclose(r_dev.cpu().numpy(), r_host, atol=1e-7, rtol=1e-6)
+    z, pq = f32(1003, seed=3, scale=4.0), np.asarray([0.4, -0.3], np.float32)
+    want = np.empty_like(z)
+    for kind, name in ((1, "silu"), (2, "gelu_tanh"), (3, "xielu")):
+        lib.sbp_activate(ptr(want), ptr(z), ctypes.c_size_t(1003), C(kind), ptr(pq))
+        assert np.allclose(ops.activate(dev(z), F32, name, dev(pq)).cpu().numpy(), want, atol=2e-6, rtol=2e-6), name
+    # recurrence, serial and in chunks
+    width = 200
+    p = f32(300, 3 * width, seed=5, scale=2.0)
+    cu, slots = i32([0, 70, 300]), i32([2, 0])
+    s_host = f32(3, width, seed=6)
+    s_serial, s_chunks = dev(s_host.copy()), dev(s_host.copy())
+    want = np.empty((300, width), np.float32)
+    assert lib.sbp_mingru_scan(ptr(want), ptr(p), ptr(s_host), ptr(cu), ptr(slots), C(2), C(width)) == 0
+    got = ops.mingru_scan(dev(p), s_serial, dev(cu), dev(slots), 2, F32)
+    assert np.allclose(got.cpu().numpy(), want, atol=2e-6, rtol=2e-6) and np.allclose(s_serial.cpu().numpy(), s_host, atol=2e-6)
+    from sonicboom_amd.engine.step import row_runs
+    chunks = dev(row_runs([70, 230], cu, ops.mingru_chunk_rows()))
+    got = ops.mingru_scan(dev(p), s_chunks, dev(cu), dev(slots), 2, F32, chunks)
+    assert np.allclose(got.cpu().numpy(), want, atol=1e-5, rtol=1e-5) and np.allclose(s_chunks.cpu().numpy(), s_host, atol=1e-5)
+    # latent attention: prepare, per-head product, attention
+    heads, dim, rot_dim, dims, rank, scale, window = 3, 8, 8, 6, 16, 0.3, 70
+    p, cw, inv_freq, table, pos, seq, stride, kv_off = latent_twin_setup()
+    uk = f32(heads, rank, dim, seed=7, scale=0.4)
+    qp, ql, cache, want = host_latent(lib, p, cw, inv_freq, table, pos, seq, stride, kv_off, heads, dim, rot_dim, dims, rank,
+                                      scale, window, uk)
+    cache_dev = torch.zeros((8, 64, rank + rot_dim), dtype=F32, device=DEV)
+    qp_dev, ql_dev = ops.latent_prepare(dev(p), 0, kv_off, F32, dev(cw), 1e-5, dev(inv_freq), dims, True, dev(pos), dev(seq),
+                                        cache_dev, dev(table), heads, dim, rot_dim, rank)
+    ops.head_product(qp_dev, dev(uk), ql_dev)
+    assert np.allclose(qp_dev.cpu().numpy(), qp) and np.allclose(ql_dev.cpu().numpy(), ql, atol=2e-5)
+    assert np.allclose(cache_dev.cpu().numpy(), cache, atol=2e-5)
+    got = ops.latent_attention_plain(ql_dev, cache_dev, dev(table), dev(pos), dev(seq), rank, scale, window)
+    assert np.allclose(got.cpu().numpy(), want, atol=3e-5)
