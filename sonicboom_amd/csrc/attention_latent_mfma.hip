@@ -157,7 +157,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   // staging: a half is kHalf rows of latent / 8 chunks of 16 bytes; thread (key = idx % kHalf, chunk = idx / kHalf)
   const int chunks = latent / 8;
   constexpr int kMaxStage = (KQ * 32 / 8 * kHalf + kAttnThreads - 1) / kAttnThreads;
-  uint4 staged[kMaxStage];
+  uint4 set_a[kMaxStage], set_b[kMaxStage];      // two halves on their way from memory to LDS
   int h_first = lo_blk / kHalf, h_last = hi_blk / kHalf;                // halves count from the sequence's start
   if (n_splits > 1) {                                                   // this block's share of them
     const int per = (h_last - h_first + n_splits) / n_splits;
@@ -169,7 +169,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
     const int p = c < max_pages ? page_table[size_t(seq) * max_pages + c] : -1;
     return (p >= 0 && p < n_pages_total) ? p : -1;
   };
-  auto load_half = [&](int h) {
+  auto load_half = [&](int h, uint4 (&staged)[kMaxStage]) {
     const int page = page_of(h);
     const bf16_t *src = cache + (size_t(max(page, 0)) * SB_PAGE + (h % (SB_PAGE / kHalf)) * kHalf) * latent;
 #pragma unroll
@@ -184,7 +184,7 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
   // what it holds (two DPP moves inside the quad) and each writes four whole 32-bit words, (even
   // key, odd key) of one number each: the even lane numbers 0 to 3 of the chunk, the odd lane 4 to 7.
   // (Written as single 16-bit stores, two lanes a word, this step took as long as all the products.)
-  auto store_half = [&](int b) {
+  auto store_half = [&](int b, const uint4 (&staged)[kMaxStage]) {
     bf16_t *ks = ks_base + b * ks_size;
     uint32_t *vt32 = reinterpret_cast<uint32_t *>(vt_base + b * vt_size);
     const bool even = (lane & 1) == 0;
@@ -212,18 +212,26 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
     }
   };
 
-  int h = h_first;
-  while (h <= h_last && page_of(h) < 0) ++h;          // pages that are not there hold no visible key
+  // Halves h (being worked on, in LDS buffer buf), h1 (on its way, in the set `held`) and h2 (asked for
+  // now, into the set `free`): a half's loads go out two steps before its rows are stored, so that
+  // they have a whole step of products and a step of stores to land.
+  auto next_half = [&](int h) -> int {
+    ++h;
+    while (h <= h_last && page_of(h) < 0) ++h;        // pages that are not there hold no visible key
+    return h;
+  };
+  int h = next_half(h_first - 1), h1 = h_last + 1;
   int buf = 0;
   if (h <= h_last) {
-    load_half(h);
-    store_half(0);
+    load_half(h, set_a);
+    store_half(0, set_a);
+    h1 = next_half(h);
+    if (h1 <= h_last) load_half(h1, set_a);
   }
   __syncthreads();                                    // the pads and the first half are written
-  while (h <= h_last) {
-    int h_next = h + 1;
-    while (h_next <= h_last && page_of(h_next) < 0) ++h_next;
-    if (h_next <= h_last) load_half(h_next);          // in flight while this half is worked on
+  auto step = [&](uint4 (&held)[kMaxStage], uint4 (&free)[kMaxStage]) {
+    const int h2 = h1 <= h_last ? next_half(h1) : h1;
+    if (h2 <= h_last) load_half(h2, free);
 
     if (wave_works) {
       const bf16_t *ks = ks_base + buf * ks_size, *vt = vt_base + buf * vt_size;
@@ -284,10 +292,16 @@ latent_attention_mfma_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict_
       }
     }
     // nobody reads the other buffer any more: its readers passed the barrier that ended the step before
-    if (h_next <= h_last) store_half(buf ^ 1);
-    __syncthreads();                                  // (after the stores: the loads they wait for have had the step's products to land)
+    if (h1 <= h_last) store_half(buf ^ 1, held);
+    __syncthreads();
     buf ^= 1;
-    h = h_next;
+    h = h1;
+    h1 = h2;
+  };
+  while (h <= h_last) {
+    step(set_a, set_b);
+    if (h > h_last) break;
+    step(set_b, set_a);
   }
 
   if (!wave_works) return;
