@@ -32,6 +32,7 @@ struct Args {
   const void *bias;
   int bias_dtype;
   const float *resid;
+  float resid_scale;   // Y = resid_scale * (X W^T + bias) + resid  (1 unless a branch has a multiplier)
   int n_rows, n_out, n_in;
   int gated;       // an sb_gate; not 0: W is [2*n_out, n_in], rows n (gate) and n_out + n (up)
   int tiles_m, tiles_n;
@@ -124,7 +125,7 @@ __device__ __forceinline__ void store_tile(const Args &a, float *lds_f, int t0, 
         if (resid) {
           const floatx4_t rv = *reinterpret_cast<const floatx4_t *>(resid + idx);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = v[q] + rv[q];
+          for (int q = 0; q < 4; ++q) v[q] = v[q] * a.resid_scale + rv[q];
         }
         if (f32_out) {
           *reinterpret_cast<floatx4_t *>(y_f + idx) = v;
@@ -140,7 +141,7 @@ __device__ __forceinline__ void store_tile(const Args &a, float *lds_f, int t0, 
           if (n_first + q >= a.n_out) continue;
           float u = v[q];
           if (bias) u = u + ld_dyn(bias, a.bias_dtype, n_first + q);
-          if (resid) u = u + resid[idx + q];
+          if (resid) u = u * a.resid_scale + resid[idx + q];
           if (f32_out) y_f[idx + q] = u;
           else y_h[idx + q] = f32_to_bf16(u);
         }
@@ -760,9 +761,22 @@ int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok, doubl
 // Y = X W^T (+bias) (+resid), or gated: Y = silu(X Wg^T) * (X Wu^T), W = [Wg; Wu].
 // X [n_rows, n_in] and W bf16, n_in a multiple of 8, operands 16-byte aligned; packed != 0: W is
 // in the packed tile layout.
+extern "C" int sb_gemm_mfma_scaled_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
+                                        int bias_dtype, const float *resid, float resid_scale, int n_rows, int n_out,
+                                        int n_in, int gated, int packed, int tile_shape, void *stream);
+
 extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                  int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
                                  int gated, int packed, int tile_shape, void *stream) {
+  return sb_gemm_mfma_scaled_bf16(y, y_dtype, x, w, bias, bias_dtype, resid, 1.0f, n_rows, n_out, n_in, gated, packed,
+                                  tile_shape, stream);
+}
+
+// The same with a multiplier on the product before the residual joins: Y = resid_scale * (X W^T + bias) + resid
+// (a multiplier of 1 gives the bits of the form above).
+extern "C" int sb_gemm_mfma_scaled_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
+                                        int bias_dtype, const float *resid, float resid_scale, int n_rows, int n_out,
+                                        int n_in, int gated, int packed, int tile_shape, void *stream) {
   SB_REQUIRE(y && x && w, "sb_gemm_mfma_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_mfma_bf16: bad sizes rows=%d out=%d in=%d",
              n_rows, n_out, n_in);
@@ -776,7 +790,7 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   if (n_rows == 0) return SB_OK;
   Args a;
   a.y = y; a.y_dtype = y_dtype; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
-  a.bias = bias; a.bias_dtype = bias_dtype; a.resid = resid;
+  a.bias = bias; a.bias_dtype = bias_dtype; a.resid = resid; a.resid_scale = resid_scale;
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated;
   a.partial = nullptr; a.stages_per_slice = 0;
   a.vec4 = n_out % 4 == 0 && (reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(resid)) % 16 == 0;
@@ -908,7 +922,7 @@ extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const vo
   if (n_rows == 0) return SB_OK;
   Args a;
   a.y = nullptr; a.y_dtype = SB_F32; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
-  a.bias = nullptr; a.bias_dtype = 0; a.resid = nullptr;
+  a.bias = nullptr; a.bias_dtype = 0; a.resid = nullptr; a.resid_scale = 1.0f;
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = 0;
   const PartialPlan plan = partial_plan(n_rows, n_out, n_in, packed && n_in % 64 == 0);
   const int tile = plan.big ? 256 : 128;

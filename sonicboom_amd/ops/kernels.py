@@ -602,6 +602,25 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     return out
 
 
+def gemm_bf16_add_scaled(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], resid: torch.Tensor,
+                         scale: float, packed_shape) -> bool:
+    """resid += scale * (x w^T (+ bias)) in the tiled product's own epilogue (packed bfloat16 weights,
+    more rows than the weight-streaming kernels take); False when the sizes are not the tiled kernel's,
+    and the caller adds in a pass of its own."""
+    _dev(x, w, bias, resid)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or packed_shape is None or x.dim() != 2:
+        return False
+    n, k = packed_shape
+    t = x.shape[0]
+    if t <= STREAM_MAX_ROWS or x.shape[1] != k or k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16:
+        return False
+    if resid.dtype != torch.float32 or tuple(resid.shape) != (t, n) or (bias is not None and bias.numel() != n):
+        raise KernelLibraryError("the residual must be float32 and shaped like the product")
+    check(library.core().sb_gemm_mfma_scaled_bf16(_p(resid), 0, _p(x), _p(w), _p(bias), _dt(bias) if bias is not None else 0,
+                                                  _p(resid), float(scale), t, n, k, 0, 1, _hints.tile_shape, _stream()))
+    return True
+
+
 @contextlib.contextmanager
 def gemm_tile_shape(shape: Optional[int], path: Optional[str] = None):
     """For tests and measurements: inside the block the tiled products of this thread use tile

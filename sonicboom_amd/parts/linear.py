@@ -85,8 +85,9 @@ class Linear:
                                          scale=scale, groups=groups)
         if scale == 1.0:
             self(x, torch.float32, resid=resid, out=resid)
-        else:
-            ops.add_scaled(resid, self(x, torch.float32), scale)
+        elif self.packed is None or x.dtype != torch.bfloat16 or not ops.gemm_bf16_add_scaled(
+                x, self.packed, self.bias, resid, scale, (self.rows, self.n_in)):
+            ops.add_scaled(resid, self(x, torch.float32), scale)      # a pass of its own over the stream
         return None
 
     def gated_product(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

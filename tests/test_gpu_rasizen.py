@@ -590,3 +590,20 @@ def test_matrix_core_latent_attention_equals_the_plain_kernel(heads, dim, rot_di
     for a, b in zip(outs[True], outs[False]):
         part_close(a, b.float().cpu().numpy(), "bfloat16", "matrix-core against plain")
     part_close(outs[True][1], outs[True][0].float().cpu().numpy(), "bfloat16", "portions and single rows against whole")
+
+
+@pytest.mark.parametrize("rows, n_out, n_in", [(300, 96, 64), (1000, 520, 256), (129, 40, 72)])
+def test_tiled_product_adds_into_the_stream_with_a_multiplier(rows, n_out, n_in):
+    """resid += scale * (x W^T + b) in the tiled product's epilogue, against the product followed by the scaled add."""
+    from sonicboom_amd import ops
+    x, w, b = rand(rows, n_in).to(BF16), rand(n_out, n_in, scale=0.2, seed=1).to(BF16), rand(n_out, seed=2)
+    resid = rand(rows, n_out, seed=3)
+    got = resid.to(DEV)
+    assert ops.gemm_bf16_add_scaled(x.to(DEV), ops.pack_weight(w.to(DEV)), b.to(DEV), got, 0.3, (n_out, n_in))
+    want = resid.numpy().astype(np.float64) + 0.3 * (x.float().numpy().astype(np.float64) @ w.float().numpy().astype(np.float64).T + b.numpy())
+    assert np.abs(got.cpu().numpy() - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+    # a multiplier of one gives the bits of the product's plain residual form
+    one, plain = resid.to(DEV), resid.to(DEV)
+    assert ops.gemm_bf16_add_scaled(x.to(DEV), ops.pack_weight(w.to(DEV)), b.to(DEV), one, 1.0, (n_out, n_in))
+    ops.gemm_bf16(x.to(DEV), ops.pack_weight(w.to(DEV)), b.to(DEV), plain, F32, plain, packed_shape=(n_out, n_in))
+    assert torch.equal(one, plain)
