@@ -7,7 +7,8 @@ per-sequence state of fixed size.
 * Cache entries (one per mixer that stores keys) with the same needs
   (kv heads, head size, window) form a **group** with storage and a page pool
   of its own: ``K: [entries, pages, kv_heads, PAGE, head_dim]`` and ``V`` with
-  the last two axes swapped.  A mixer may keep something else per token instead:
+  the last two axes swapped (and ``v_dim`` in place of ``head_dim`` where a mixer's
+  values have a size of their own).  A mixer may keep something else per token instead:
   rows of a shape of its own, ``[entries, pages, PAGE, *shape]``, in groups by
   (shape, window).  A group
   that only reads a window of keys gives pages back as the window leaves them.
@@ -79,6 +80,7 @@ class GroupSpec:
     window: int                  # 0: every key is kept
     entries: Tuple[int, ...]     # cache entry numbers stored in this group
     row_shape: Tuple[int, ...] = ()   # not empty: a row of this shape per token instead of keys and values
+    v_dim: int = 0               # the values' size per head when it is not head_dim (0: the same)
 
 
 @dataclass
@@ -135,7 +137,7 @@ class PagedCache:
                 # keys [.., position, d]; values transposed [.., d, position] (see csrc/sb_hip.h)
                 self.k.append(torch.zeros((n, pages, spec.kv_heads, PAGE, spec.head_dim),
                                           dtype=dtype, device=device))
-                self.v.append(torch.zeros((n, pages, spec.kv_heads, spec.head_dim, PAGE),
+                self.v.append(torch.zeros((n, pages, spec.kv_heads, spec.v_dim or spec.head_dim, PAGE),
                                           dtype=dtype, device=device))
             for key, (shape, sdtype) in (state_shapes or {}).items():
                 self.state[key] = torch.zeros((self.max_slots, *shape), dtype=sdtype, device=device)
@@ -291,10 +293,14 @@ class PagedCache:
 
 
 def group_entries(specs: Dict[int, tuple]) -> List[GroupSpec]:
-    """Group cache entries {entry: (kv_heads, head_dim, window)}, or {entry: ("rows", shape, window)}
-    for entries that keep a row of their own shape per token, by equal needs, in order of first use."""
+    """Group cache entries {entry: (kv_heads, head_dim, window[, values' size])}, or {entry: ("rows",
+    shape, window)} for entries that keep a row of their own shape per token, by equal needs, in order
+    of first use."""
     by_need: Dict[tuple, List[int]] = {}
     for e in sorted(specs):
         by_need.setdefault(tuple(specs[e]), []).append(e)
-    return [GroupSpec(0, 0, k[2], tuple(v), tuple(k[1])) if k[0] == "rows" else GroupSpec(k[0], k[1], k[2], tuple(v))
+    def values_size(k):
+        return k[3] if len(k) > 3 and k[3] != k[1] else 0
+    return [GroupSpec(0, 0, k[2], tuple(v), tuple(k[1])) if k[0] == "rows"
+            else GroupSpec(k[0], k[1], k[2], tuple(v), v_dim=values_size(k))
             for k, v in by_need.items()]

@@ -28,7 +28,8 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
                        const TC *__restrict__ k_cache, const TC *__restrict__ v_cache,
                        const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                        const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
-                       int heads_q, int heads_kv, int head_dim, float scale, int window) {
+                       int heads_q, int heads_kv, int head_dim, float scale, int window, int v_dim,
+                       float softcap, int sink) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[64];
   const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -39,15 +40,16 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
 
   const int lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const float neg_inf = -__builtin_inff();
-  float m = neg_inf, l = 0.0f;
+  // a sink is one more key of score 0 that has no value: the running maximum starts at its score
+  // and the running sum at its weight
+  float m = sink ? 0.0f : neg_inf, l = sink ? 1.0f : 0.0f;
   float o[kMaxHeadDim / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
 
   for (int c = lo / SB_PAGE; c <= pos / SB_PAGE; ++c) {
     const int page = c < max_pages ? page_table[size_t(seq) * max_pages + c] : -1;
     if (page < 0 || page >= n_pages_total) continue;  // uniform over the wave
-    const size_t base = (size_t(page) * heads_kv + kvh) * SB_PAGE * head_dim;
-    const TC *kp = k_cache + base;
-    const TC *vp = v_cache + base;
+    const TC *kp = k_cache + (size_t(page) * heads_kv + kvh) * SB_PAGE * head_dim;
+    const TC *vp = v_cache + (size_t(page) * heads_kv + kvh) * SB_PAGE * v_dim;
     const int j = c * SB_PAGE + lane;
     const bool visible = j >= lo && j <= pos;
     float s = neg_inf;
@@ -55,6 +57,7 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
       float dot = 0.0f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], ld_f(kp, sb_key_index(lane, d, head_dim)), dot);
       s = dot * scale;
+      if (softcap > 0.0f) s = softcap * tanhf(s / softcap);
     }
     const float cm = wave_max(s);
     const float m_new = fmaxf(m, cm);
@@ -67,7 +70,7 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
 #pragma unroll
     for (int i = 0; i < kMaxHeadDim / 64; ++i) {
       const int d = lane + 64 * i;
-      if (d < head_dim) {
+      if (d < v_dim) {
         float acc = o[i] * alpha;
         for (int jj = j0; jj <= j1; ++jj) acc = fmaf(ps[jj], ld_f(vp, sb_value_index(d, jj)), acc);
         o[i] = acc;
@@ -80,17 +83,39 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
 #pragma unroll
   for (int i = 0; i < kMaxHeadDim / 64; ++i) {
     const int d = lane + 64 * i;
-    if (d < head_dim) st_f(out, size_t(row) * heads_q * head_dim + size_t(h) * head_dim + d, o[i] * inv);
+    if (d < v_dim) st_f(out, size_t(row) * heads_q * v_dim + size_t(h) * v_dim + d, o[i] * inv);
   }
 }
 
 }  // namespace
+
+// The same with values of another size than the keys (v_dim; the cache then holds values
+// [page][kv head][v_dim][position] and out is [rows, heads_q * v_dim]), scores capped as
+// softcap * tanh(s / softcap) when softcap > 0, and with `sink` one more key of score 0 without a
+// value in every row's softmax: weights exp(s_j) / (1 + sum exp(s_j)).
+extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                                   const void *v_cache, int cache_dtype, const int32_t *page_table,
+                                   int max_pages, int n_pages_total, const int32_t *row_pos,
+                                   const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
+                                   int head_dim, int v_dim, float scale, int window, float softcap, int sink,
+                                   void *stream);
 
 extern "C" int sb_attention(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
                             const void *v_cache, int cache_dtype, const int32_t *page_table,
                             int max_pages, int n_pages_total, const int32_t *row_pos,
                             const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
                             int head_dim, float scale, int window, void *stream) {
+  return sb_attention_capped(out, q, act_dtype, q_stride, k_cache, v_cache, cache_dtype, page_table, max_pages,
+                             n_pages_total, row_pos, row_seq, n_rows, heads_q, heads_kv, head_dim, head_dim, scale,
+                             window, 0.0f, 0, stream);
+}
+
+extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                                   const void *v_cache, int cache_dtype, const int32_t *page_table,
+                                   int max_pages, int n_pages_total, const int32_t *row_pos,
+                                   const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
+                                   int head_dim, int v_dim, float scale, int window, float softcap, int sink,
+                                   void *stream) {
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && row_seq,
              "sb_attention: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads_q > 0 && heads_kv > 0 && head_dim > 0 && max_pages > 0 &&
@@ -102,8 +127,9 @@ extern "C" int sb_attention(void *out, const void *q, int act_dtype, int q_strid
   SB_REQUIRE(q_stride >= heads_q * head_dim, "sb_attention: query stride %d shorter than %d", q_stride,
              heads_q * head_dim);
   SB_REQUIRE(sb::valid_dtype(act_dtype) && sb::valid_dtype(cache_dtype), "sb_attention: unknown dtype");
-  SB_SUPPORT(head_dim <= kMaxHeadDim, "sb_attention: head size %d is above the limit of %d", head_dim,
-             kMaxHeadDim);
+  SB_SUPPORT(head_dim <= kMaxHeadDim && v_dim > 0 && v_dim <= kMaxHeadDim,
+             "sb_attention: head sizes %d and %d must be positive and at most %d", head_dim, v_dim, kMaxHeadDim);
+  SB_REQUIRE(softcap >= 0.0f, "sb_attention: the cap of the scores must not be negative");
   SB_SUPPORT(heads_q <= 65535, "sb_attention: more than 65535 query heads");
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
@@ -111,7 +137,8 @@ extern "C" int sb_attention(void *out, const void *q, int act_dtype, int q_strid
 #define SB_GO(TA, TC)                                                                           \
   attention_plain_kernel<TA, TC><<<grid, 64, 0, s>>>(                                            \
       (TA *)out, (const TA *)q, q_stride, (const TC *)k_cache, (const TC *)v_cache, page_table,  \
-      max_pages, n_pages_total, row_pos, row_seq, heads_q, heads_kv, head_dim, scale, window)
+      max_pages, n_pages_total, row_pos, row_seq, heads_q, heads_kv, head_dim, scale, window, v_dim,  \
+      softcap, sink)
   if (act_dtype == SB_F32 && cache_dtype == SB_F32) SB_GO(float, float);
   else if (act_dtype == SB_BF16 && cache_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
   else if (act_dtype == SB_F32 && cache_dtype == SB_BF16) SB_GO(float, bf16_t);

@@ -31,10 +31,20 @@ __device__ __forceinline__ void st_f(bf16_t *p, size_t i, float v) { p[i] = f32_
 // SB_GATE_SILU g / (1 + exp(-g)) with the full-precision expf
 // (/root/reference/core/src/nn/activation.cpp:41-50); SB_GATE_GELU_TANH the tanh form of GELU,
 // 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))), constants and order of :27-36.
+// SB_GATE_RELU max(g, 0).
 __device__ __forceinline__ float gate_act(float g, int kind) {
+  if (kind == SB_GATE_RELU) return fmaxf(g, 0.0f);
   if (kind == SB_GATE_GELU_TANH)
     return 0.5f * g * (1.0f + tanhf(0.79788456080286535587989211986876f * g * (1.0f + 0.044715f * g * g)));
   return g / (1.0f + expf(-g));
+}
+
+// The clamped swish pair of an expert: g' = min(g, limit), u' = u cut to [-limit, limit];
+// g' sigmoid(alpha g') (u' + 1).
+__device__ __forceinline__ float swish_clamp_mul(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return (g / (1.0f + expf(-alpha * g))) * (u + 1.0f);
 }
 
 // The rotation of one pair (x0, x1) by the angle whose cosine and sine are c and s: every product

@@ -41,7 +41,7 @@ extern "C" int sb_gate_mul(void *out, int out_dtype, const void *gu, int gu_dtyp
   SB_REQUIRE(out && gu, "sb_gate_mul: null pointer");
   SB_REQUIRE(n_rows >= 0 && width > 0, "sb_gate_mul: bad sizes rows=%d width=%d", n_rows, width);
   SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(gu_dtype), "sb_gate_mul: unknown dtype");
-  SB_SUPPORT(gate == SB_GATE_SILU || gate == SB_GATE_GELU_TANH, "sb_gate_mul: unknown gate activation %d", gate);
+  SB_SUPPORT(gate >= SB_GATE_SILU && gate <= SB_GATE_RELU, "sb_gate_mul: unknown gate activation %d", gate);
   const size_t total = size_t(n_rows) * width;
   if (total == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
@@ -201,4 +201,19 @@ extern "C" int sb_read_probe(void *sink, const void *src, size_t bytes, int bloc
   SB_REQUIRE(sink && src && blocks > 0, "sb_read_probe: bad arguments");
   read_probe_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((uint32_t *)sink, (const uint4 *)src, bytes / 16);
   return sb::check_launch("sb_read_probe");
+}
+
+// ---- a multiplier on float32 values in place (the logits of a head that has one) ---------------
+namespace {
+__global__ void scale_kernel(float *__restrict__ x, float scale, size_t n) {
+  const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) x[i] = x[i] * scale;
+}
+}  // namespace
+
+extern "C" int sb_scale(float *x, float scale, size_t n, void *stream) {
+  SB_REQUIRE(x || n == 0, "sb_scale: null pointer");
+  if (n == 0) return SB_OK;
+  scale_kernel<<<unsigned((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, scale, n);
+  return sb::check_launch("sb_scale");
 }

@@ -672,6 +672,8 @@ int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
   // the gate's activation is a template argument: the SiLU kernels hold no code of the others
   const int which = a.gated * 4 + (packed ? 2 : 0) + (a.n_in % BK == 0 ? 1 : 0);
   switch (which) {
+    case 15: return launch_one<MT, NW, BK, DEPTH, 3, true, true>(a, blocks, s);
+    case 14: return launch_one<MT, NW, BK, DEPTH, 3, true, false>(a, blocks, s);
     case 11: return launch_one<MT, NW, BK, DEPTH, 2, true, true>(a, blocks, s);
     case 10: return launch_one<MT, NW, BK, DEPTH, 2, true, false>(a, blocks, s);
     case 7: return launch_one<MT, NW, BK, DEPTH, 1, true, true>(a, blocks, s);
@@ -682,6 +684,8 @@ int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
   }
   if constexpr (PLAIN_TOO) {
     switch (which) {
+      case 13: return launch_one<MT, NW, BK, DEPTH, 3, false, true>(a, blocks, s);
+      case 12: return launch_one<MT, NW, BK, DEPTH, 3, false, false>(a, blocks, s);
       case 9: return launch_one<MT, NW, BK, DEPTH, 2, false, true>(a, blocks, s);
       case 8: return launch_one<MT, NW, BK, DEPTH, 2, false, false>(a, blocks, s);
       case 5: return launch_one<MT, NW, BK, DEPTH, 1, false, true>(a, blocks, s);
@@ -718,6 +722,7 @@ int launch_direct_one(const Args &a, long long blocks, int round_blocks, hipStre
 template <int MT16, int NW, int BK, int NBUF, bool PERSIST>
 int launch_direct(const Args &a, long long blocks, int round_blocks, hipStream_t s) {
   switch (a.gated) {
+    case 3: return launch_direct_one<MT16, NW, BK, NBUF, 3, PERSIST>(a, blocks, round_blocks, s);
     case 2: return launch_direct_one<MT16, NW, BK, NBUF, 2, PERSIST>(a, blocks, round_blocks, s);
     case 1: return launch_direct_one<MT16, NW, BK, NBUF, 1, PERSIST>(a, blocks, round_blocks, s);
     default: return launch_direct_one<MT16, NW, BK, NBUF, 0, PERSIST>(a, blocks, round_blocks, s);
@@ -786,7 +791,7 @@ extern "C" int sb_gemm_mfma_scaled_bf16(void *y, int y_dtype, const void *x, con
   SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
              "sb_gemm_mfma_bf16: operands must be 16-byte aligned");
   SB_REQUIRE(!(gated && (bias || resid)), "sb_gemm_mfma_bf16: the gated form takes no bias or residual");
-  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_mfma_bf16: unknown gate activation %d", gated);
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_RELU, "sb_gemm_mfma_bf16: unknown gate activation %d", gated);
   if (n_rows == 0) return SB_OK;
   Args a;
   a.y = y; a.y_dtype = y_dtype; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;

@@ -284,7 +284,7 @@ extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const vo
   SB_REQUIRE(need == 0 || (scratch && scratch_floats >= need),
              "sb_gemm_skinny_bf16: scratch of %zu floats needed, %zu given", need, scratch_floats);
   hipStream_t s = (hipStream_t)stream;
-  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_skinny_bf16: unknown gate activation %d", gated);
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_RELU, "sb_gemm_skinny_bf16: unknown gate activation %d", gated);
   Epilogue ep{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, gated};
   float *partial = p.n_slices > 1 ? scratch : nullptr;
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;

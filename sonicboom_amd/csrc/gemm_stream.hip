@@ -297,7 +297,7 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
              "sb_gemm_stream_bf16: inner size %d is too large", n_in);
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_stream_bf16: unknown gate activation %d", gated);
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_RELU, "sb_gemm_stream_bf16: unknown gate activation %d", gated);
   const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in, nullptr, 0, gated};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   const int tt = row_tiles(n_rows);

@@ -71,7 +71,7 @@ typedef enum sb_dtype { SB_F32 = 0, SB_BF16 = 1 } sb_dtype;
 
 /* The `gated` argument of the products and of sb_gate_mul: not gated, or the activation of the
  * gate in Y = act(X Wg^T) * (X Wu^T). */
-typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2 } sb_gate;
+typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2, SB_GATE_RELU = 3 } sb_gate;
 
 /* The `kind` argument of sb_activate.  xIELU takes two numbers (p, q) from memory: for z > 0
  * softplus(p) z^2 + z/2, else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */

@@ -73,14 +73,14 @@ class DecoderModel:
                 cs = mixer.cache_spec()
                 if cs is None:
                     raise ValueError(f"order entry {i} names cache {e.cache} but its mixer keeps no keys")
-                need = cs.key()          # (kv heads, head size, window), or ("rows", shape, window)
+                need = cs.key()          # (kv heads, head size, window, values' size), or ("rows", shape, window)
                 have = self.cache_specs.get(e.cache)
-                if have is not None and have[:2] != need[:2]:
+                if have is not None and have[:2] + have[3:] != need[:2] + need[3:]:
                     raise ValueError(f"order entry {i} uses cache {e.cache} whose heads (or rows) differ from its own")
                 if have is not None:
                     # the entry keeps what its widest reader sees: every key if one of them has no
                     # window, else the largest window of all that read it
-                    need = need[:2] + (0 if 0 in (have[2], need[2]) else max(have[2], need[2]),)
+                    need = need[:2] + (0 if 0 in (have[2], need[2]) else max(have[2], need[2]),) + need[3:]
                 self.cache_specs[e.cache] = need
             ss = mixer.state_spec()
             if ss is not None:

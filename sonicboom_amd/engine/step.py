@@ -112,6 +112,7 @@ class _Context:
     """What the parts read of a step's bookkeeping (see :class:`StepContext`)."""
 
     trace = None            # set by the engine while a tracer listens
+    shared = None           # a step's own scratch: what a part leaves for a later part of the same step
 
     def page_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
@@ -309,6 +310,7 @@ class Engine:
         their run order, and for the wanted rows the final norm and the head."""
         model = self.model
         tracer = self.tracer
+        ctx.shared = {}
         x = model.embedding.forward(ctx.ids, ctx)
         if tracer is not None:
             tracer("embedding", x)
@@ -320,6 +322,7 @@ class Engine:
             ctx.trace = (lambda what, t, _i=i: tracer(f"entry{_i}.{what}", t)) if tracer is not None else None
             h = model.blocks[e.block].forward(x, ctx, self.bindings[i], h=h, next_norm=next_norm)
         ctx.trace = None
+        ctx.shared = None
         if ctx.n_wanted == 0:
             return torch.empty((0, model.vocab), dtype=torch.float32, device=self.device)
         h = model.final_norm.forward(x, model.rt.act_dtype, rows=ctx.want_rows)

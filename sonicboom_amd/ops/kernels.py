@@ -141,7 +141,7 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], r
     return out
 
 
-GATES = {"silu": 1, "gelu_tanh": 2}      # sb_gate of csrc/sb_hip.h
+GATES = {"silu": 1, "gelu_tanh": 2, "relu": 3}      # sb_gate of csrc/sb_hip.h
 
 
 def gate_code(activation) -> int:
@@ -1046,3 +1046,280 @@ def latent_attention(q: torch.Tensor, cache: torch.Tensor, page_table: torch.Ten
                                      window, single_rows=bool(ctx.is_decode),
                                      max_keys=min(keys, window) if window > 0 else keys)
     return latent_attention_plain(q, cache, page_table, ctx.row_pos, ctx.row_seq, rank, scale, window)
+
+
+# --------------------------------------------------------------------------
+# norms of what leaves a sublayer; an embedding with positions; head norms; capped attention; experts
+# --------------------------------------------------------------------------
+def offset_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, offset: float, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * (offset + weight) of float32 rows ``x`` [n, width]; ``rows``
+    (int32) picks and orders source rows."""
+    _dev(x, weight, rows)
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise KernelLibraryError("the norm's input must be float32 [rows, width]")
+    width = x.shape[1]
+    if weight is not None and weight.numel() != width:
+        raise KernelLibraryError(f"the norm's weight has {weight.numel()} elements, the rows have {width}")
+    n = x.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "row index")
+    y = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    check(library.core().sb_offset_norm(_p(y), _dt(y), _p(x), _p(weight), _dt(weight) if weight is not None else 0,
+                                        _p(rows), n, width, float(eps), float(offset), _stream()))
+    return y
+
+
+def norm_add(x: torch.Tensor, part: torch.Tensor, weight: Optional[torch.Tensor], eps: float, offset: float,
+             copy_dtype: Optional[torch.dtype] = None, part_weights: Optional[torch.Tensor] = None,
+             extra: Optional[torch.Tensor] = None, extra_weights: Optional[torch.Tensor] = None,
+             by_row: bool = False, norm: bool = True) -> Optional[torch.Tensor]:
+    """x += un(sum_s a_s part_s (+ b extra)), un(v) = v / sqrt(mean(v^2) + eps) * (offset + weight)
+    (``norm`` false: the sum as it is); returns the new x in ``copy_dtype`` when that is given.
+
+    ``part`` float32 [rows, width], or slices of it: [slices, rows, width], or with ``by_row``
+    [rows, slices, width].  ``part_weights`` (float32, a view [rows, slices] of rows that may be
+    longer): the multiplier a_s of every row's slices, else 1.  ``extra`` float32 [rows, width] with
+    ``extra_weights`` (a view [rows] or [rows, 1]) one multiplier a row."""
+    _dev(x, part, weight, extra)
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise KernelLibraryError("the stream must be float32 [rows, width]")
+    n, width = x.shape
+    if part.dtype != torch.float32:
+        raise KernelLibraryError("the sublayer's result must be float32")
+    if part.dim() == 2:
+        part = part.view(1, n, width)
+        by_row = False
+    if part.dim() != 3 or part.shape[2] != width or part.shape[0 if by_row else 1] != n:
+        raise KernelLibraryError(f"the sublayer's result {tuple(part.shape)} does not fit the stream {tuple(x.shape)}")
+    slices = part.shape[1 if by_row else 0]
+    slice_stride, row_stride = (width, slices * width) if by_row else (n * width, width)
+    pw_stride = ew_stride = 0
+    for t, what in ((part_weights, "slice"), (extra_weights, "row")):
+        if t is not None and (t.dtype != torch.float32 or not t.is_cuda or t.shape[0] != n or t.stride(-1) != 1):
+            raise KernelLibraryError(f"the {what} multipliers must be float32 rows on the GPU")
+    if part_weights is not None:
+        if part_weights.dim() != 2 or part_weights.shape[1] != slices:
+            raise KernelLibraryError("one multiplier for every slice of every row")
+        pw_stride = part_weights.stride(0)
+    if extra is not None:
+        if extra.dtype != torch.float32 or tuple(extra.shape) != (n, width):
+            raise KernelLibraryError("the extra addend must be float32 and shaped like the stream")
+        if extra_weights is not None:
+            ew_stride = extra_weights.stride(0)
+    if weight is not None and weight.numel() != width:
+        raise KernelLibraryError(f"the norm's weight has {weight.numel()} elements, the rows have {width}")
+    copy = None
+    if copy_dtype is not None and copy_dtype != torch.float32:
+        copy = torch.empty((n, width), dtype=copy_dtype, device=x.device)
+    check(library.core().sb_norm_add(
+        _p(x), _p(copy), _dt(copy) if copy is not None else 0, _p(part), slices, slice_stride, row_stride,
+        _p(part_weights), pw_stride, _p(extra), _p(extra_weights) if extra is not None else None, ew_stride,
+        _p(weight), _dt(weight) if weight is not None else 0, n, width, float(eps), float(offset), 1 if norm else 0,
+        _stream()))
+    return x if copy_dtype == torch.float32 else copy
+
+
+def embed_pos_norm(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0, positions: Optional[torch.Tensor] = None,
+                   row_pos: Optional[torch.Tensor] = None, weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                   offset: float = 0.0, norm: bool = False, copy_dtype: Optional[torch.dtype] = None):
+    """x = table[ids] * scale (+ positions[row_pos]), then with ``norm`` x / sqrt(mean(x^2) + eps) *
+    (offset + weight); float32 [n, width], and a copy in ``copy_dtype`` when that is given (and not
+    float32).  An id or a position outside its table gives a row of NaN."""
+    _dev(table, ids, positions, row_pos, weight)
+    if table.dim() != 2 or (positions is not None and (positions.dim() != 2 or positions.shape[1] != table.shape[1])):
+        raise KernelLibraryError("the tables must be [vocab, width] and [positions, width]")
+    n = ids.numel()
+    _i32(ids, n, "token ids")
+    if positions is not None:
+        if row_pos is None:
+            raise KernelLibraryError("a table of positions needs the rows' positions")
+        _i32(row_pos, n, "row positions")
+    vocab, width = table.shape
+    if weight is not None and weight.numel() != width:
+        raise KernelLibraryError(f"the norm's weight has {weight.numel()} elements, the rows have {width}")
+    x = torch.empty((n, width), dtype=torch.float32, device=table.device)
+    copy = None
+    if copy_dtype is not None and copy_dtype != torch.float32:
+        copy = torch.empty((n, width), dtype=copy_dtype, device=table.device)
+    check(library.core().sb_embed_pos_norm(
+        _p(x), _p(copy), _dt(copy) if copy is not None else 0, _p(table), _dt(table), _p(positions),
+        _dt(positions) if positions is not None else 0, _p(ids), _p(row_pos), n, vocab,
+        positions.shape[0] if positions is not None else 0, float(scale), _p(weight),
+        _dt(weight) if weight is not None else 0, width, float(eps), float(offset), 1 if norm else 0, _stream()))
+    return x, copy
+
+
+def _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim):
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (heads_kv, PAGE, head_dim) \
+            or tuple(v_cache.shape[1:]) != (heads_kv, v_dim, PAGE) or k_cache.shape[0] != v_cache.shape[0] \
+            or k_cache.dtype != v_cache.dtype:
+        raise KernelLibraryError(
+            f"cache must be keys [pages, {heads_kv}, {PAGE}, {head_dim}] and values "
+            f"[pages, {heads_kv}, {v_dim}, {PAGE}], found {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
+
+
+def headnorm_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, q_weight: Optional[torch.Tensor],
+                      k_weight: Optional[torch.Tensor], eps: float, row_pos: torch.Tensor, row_seq: torch.Tensor,
+                      k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+                      heads_q: int, heads_kv: int, head_dim: int, v_dim: int, store: bool = True,
+                      v_first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None,
+                      v_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From float32 rows [n, heads_q*head_dim + heads_kv*(head_dim + v_dim)] of a stacked product (or
+    [slices, n, ...], added here): every head of q and k divided by its root mean square and
+    multiplied by a weight [head_dim] that the heads share (None: as it is), the values mixed as
+    (1 - lam) v + lam v_first when ``v_first`` (float32 [n, heads_kv*v_dim]) is given, the values of
+    before the mixing written to ``v_out``; returns q [n, heads_q*head_dim] in ``q_dtype`` and, with
+    ``store``, puts keys and values into the pages of the rows' positions."""
+    _dev(qkv, q_weight, k_weight, row_pos, row_seq, k_cache, v_cache, page_table, v_first, lam, v_out)
+    if qkv.dtype != torch.float32:
+        raise KernelLibraryError("the stacked product must be float32")
+    n_slices = 1
+    if qkv.dim() == 3:
+        n_slices = qkv.shape[0]
+        qkv = qkv.view(-1, qkv.shape[2])
+    n = qkv.shape[0] // n_slices
+    need = heads_q * head_dim + (heads_kv * (head_dim + v_dim) if store else 0)
+    if qkv.dim() != 2 or qkv.shape[1] < need:
+        raise KernelLibraryError(f"rows of the stacked product have {qkv.shape[1]} elements, {need} are needed")
+    for w in (q_weight, k_weight):
+        if w is not None and w.numel() != head_dim:
+            raise KernelLibraryError(f"a head norm's weight has {w.numel()} elements, a head has {head_dim}")
+    if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+        raise KernelLibraryError("the head norms' weights must be of one type")
+    wt = q_weight if q_weight is not None else k_weight
+    max_pages = n_pages = 0
+    if store:
+        _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
+        _check_rows(row_pos, row_seq, page_table, n)
+        max_pages, n_pages = page_table.shape[1], k_cache.shape[0]
+    nv = heads_kv * v_dim
+    for t, what in ((v_first, "values to mix with"), (v_out, "values to hand on")):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != n * nv):
+            raise KernelLibraryError(f"the {what} must be float32 [rows, {nv}]")
+    if v_first is not None and (lam is None or lam.numel() != 1):
+        raise KernelLibraryError("mixing values takes one number")
+    q = torch.empty((n, heads_q * head_dim), dtype=q_dtype, device=qkv.device)
+    check(library.core().sb_headnorm_kv_store(
+        _p(q), _dt(q), _p(qkv), qkv.shape[1], n_slices, _p(q_weight), _p(k_weight), _dt(wt) if wt is not None else 0,
+        float(eps), _p(v_first), _p(lam) if v_first is not None else None, _dt(lam) if lam is not None else 0, _p(v_out),
+        _p(row_pos), _p(row_seq), _p(k_cache), _p(v_cache), _dt(k_cache) if store else 0, _p(page_table), max_pages,
+        n_pages, n, heads_q, heads_kv, head_dim, v_dim, 1 if store else 0, _stream()))
+    return q
+
+
+def attention_capped_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                           row_pos: torch.Tensor, row_seq: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
+                           v_dim: int, scale: float, window: int, softcap: float, sink: bool) -> torch.Tensor:
+    """Attention of rows ``q`` [n, hq*hd] over the cache by the plain kernel, values of ``v_dim``,
+    scores capped as softcap tanh(s / softcap) (0: not), with ``sink`` one more key of score 0
+    without a value in every softmax; [n, hq*v_dim]."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, row_seq)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim:
+        raise KernelLibraryError(f"queries must be [rows, {heads_q * head_dim}]")
+    _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
+    _check_rows(row_pos, row_seq, page_table, n)
+    out = torch.empty((n, heads_q * v_dim), dtype=q.dtype, device=q.device)
+    check(library.core().sb_attention_capped(
+        _p(out), _p(q), _dt(q), q.shape[1], _p(k_cache), _p(v_cache), _dt(k_cache), _p(page_table),
+        page_table.shape[1], k_cache.shape[0], _p(row_pos), _p(row_seq), n, heads_q, heads_kv, head_dim, v_dim,
+        float(scale), int(window), float(softcap), 1 if sink else 0, _stream()))
+    return out
+
+
+def scale_(x: torch.Tensor, scale: float) -> torch.Tensor:
+    """x *= scale in place (float32)."""
+    _dev(x)
+    if x.dtype != torch.float32:
+        raise KernelLibraryError("scale_ takes float32 values")
+    check(library.core().sb_scale(_p(x), float(scale), x.numel(), _stream()))
+    return x
+
+
+MOE_MAX_TOP = 16        # choices a row that the router kernel takes (sb_moe_max_top)
+
+
+class MoEWeight:
+    """The stacked matrices of a set of experts, [experts, out (or 2 * out: gate over up), in], as
+    the experts' product kernels read them."""
+
+    def __init__(self, w: torch.Tensor, gated: bool = False, fast: bool = True):
+        if w.dim() != 3 or (gated and w.shape[1] % 2):
+            raise KernelLibraryError("experts' matrices must be stacked [experts, out, in]")
+        self.w = w.contiguous()
+        self.gated = gated
+        self.experts, rows, self.n_in = w.shape
+        self.n_out = rows // 2 if gated else rows
+        self.fast = fast
+
+
+class MoEPlan:
+    """Which expert every (row, choice) pair takes: ``ids`` int32 [pairs] (None: all take expert 0)."""
+
+    def __init__(self, ids: Optional[torch.Tensor], n_pairs: int, n_experts: int):
+        self.ids, self.n_pairs, self.n_experts = ids, n_pairs, n_experts
+
+
+def moe_plan(ids: Optional[torch.Tensor], n_experts: int, n_pairs: Optional[int] = None, device=None) -> MoEPlan:
+    if ids is not None:
+        ids = ids.view(-1)
+        n_pairs = ids.numel()
+    return MoEPlan(ids, int(n_pairs), int(n_experts))
+
+
+def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dtype: torch.dtype,
+                limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """Y[p] = X[p // x_div] W_e^T for every pair p of ``plan``; a gated weight gives the clamped
+    swish pair of its two halves."""
+    if w.experts != plan.n_experts:
+        raise KernelLibraryError(f"the plan counts {plan.n_experts} experts, the weight has {w.experts}")
+    return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha)
+
+
+def attention_capped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
+                     heads_q: int, heads_kv: int, head_dim: int, v_dim: int, scale: float, window: int,
+                     softcap: float, sink: bool, fast: bool = True) -> torch.Tensor:
+    """Attention of a step's rows over the cache with values of their own size, capped scores and a
+    sink (see :func:`attention_capped_plain`)."""
+    return attention_capped_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
+                                  head_dim, v_dim, scale, window, softcap, sink)
+
+
+def moe_max_top() -> int:
+    return int(library.core().sb_moe_max_top())
+
+
+def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool):
+    """From router scores ``z`` float32 [n, >= n_experts (+ 1)]: the ``top`` largest of the first
+    ``n_experts`` of every row (ties to the lower number) as int32 [n, top], and float32 [n, top + 1]:
+    the softmax over the chosen scores, then sigmoid(z[:, n_experts]) with ``has_gate`` (else 0)."""
+    _dev(z)
+    if z.dtype != torch.float32 or z.dim() != 2:
+        raise KernelLibraryError("router scores must be float32 [rows, experts]")
+    n = z.shape[0]
+    ids = torch.empty((n, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((n, top + 1), dtype=torch.float32, device=z.device)
+    check(library.core().sb_moe_route(_p(ids), _p(weights), _p(z), n, z.shape[1], int(n_experts), int(top),
+                                      1 if has_gate else 0, _stream()))
+    return ids, weights
+
+
+def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tensor], n_pairs: int, x_div: int,
+                      out_dtype: torch.dtype, gated: bool = False, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+    """Y[p] = X[p // x_div] W_e^T, e = ids[p] (None: expert 0), by the plain kernel.  ``w``
+    [experts, out (or 2*out, gate over up, with ``gated``), in]; gated: the clamped swish pair
+    g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = u cut to +-limit."""
+    _dev(x, w, ids)
+    if w.dim() != 3 or x.dim() != 2 or x.shape[1] != w.shape[2]:
+        raise KernelLibraryError(f"expert product shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    n_experts, rows, n_in = w.shape
+    n_out = rows // 2 if gated else rows
+    if ids is not None:
+        _i32(ids, n_pairs, "expert numbers")
+    if (n_pairs + x_div - 1) // x_div > x.shape[0]:
+        raise KernelLibraryError("more pairs than rows to take them from")
+    y = torch.empty((n_pairs, n_out), dtype=out_dtype, device=x.device)
+    check(library.core().sb_moe_product(_p(y), _dt(y), _p(x), _dt(x), _p(w), _dt(w), _p(ids), n_pairs, int(x_div),
+                                        n_out, n_in, n_experts, 1 if gated else 0, float(limit), float(alpha), _stream()))
+    return y

@@ -52,6 +52,16 @@ _CORE_SIGNATURES = {
     "sb_head_product_bf16": [_P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "sb_latent_attention_tile_rows": [],
     "sb_latent_attention_bf16_ok": [_I, _I],
+    "sb_offset_norm": [_P, _I, _P, _P, _I, _P, _I, _I, _F, _F, _P],
+    "sb_norm_add": [_P, _P, _I, _P, _I, _Z, _Z, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _F, _I, _P],
+    "sb_scale": [_P, _F, _Z, _P],
+    "sb_embed_pos_norm": [_P, _P, _I, _P, _I, _P, _I, _P, _P, _I, _I, _I, _F, _P, _I, _I, _F, _F, _I, _P],
+    "sb_headnorm_kv_store": [_P, _I, _P, _I, _I, _P, _P, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I,
+                             _I, _I, _I, _I, _I, _P],
+    "sb_attention_capped": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P],
+    "sb_moe_max_top": [],
+    "sb_moe_route": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "sb_moe_product": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }
 # Entry points of later kernels; declared when the library has them.

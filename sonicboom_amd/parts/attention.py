@@ -8,7 +8,14 @@ multiplier (/root/reference/core/src/model/recipe.cpp:65-70, :165-167).
 Every size and switch is a parameter of the spec:
 
     heads_q, heads_kv, head_dim, window (0 = all keys), scale (None = 1/sqrt),
-    qkv_bias, out_bias, out_scale (the multiplier of the branch, 1 unless given)
+    qkv_bias, out_bias, out_scale (the multiplier of the branch, 1 unless given),
+    v_dim (the values' size per head when it is not the keys'), qk_norm (every head of q and k
+    divided by its root mean square, eps ``qk_norm_eps`` inside the root, times a weight of the head's
+    size that the heads share), softcap (scores become softcap * tanh(score / softcap); 0: not),
+    sink (one more key of score 0 without a value in every softmax: the weights are
+    exp(s_j) / (1 + sum exp(s_j))), value_mix ("first": the values of this step's rows are kept
+    for later layers under ``value_mix_key``; "mix": v <- (1 - lam) v + lam v_first with the layer's
+    own number lam; what is mixed is what the cache keeps)
 
 and the position encoding is a nested part.  The three input projections are
 packed into one matrix when the mixer is built, so a step runs one product
@@ -28,26 +35,47 @@ from .linear import Linear
 from .spec import PartSpec, TensorSpec
 
 
+NAMES = {"q_weight": "q_proj.weight", "k_weight": "k_proj.weight", "v_weight": "v_proj.weight",
+         "o_weight": "o_proj.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+         "o_bias": "o_proj.bias", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
+
+
 def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_dim: int,
                    position: PartSpec, window: int = 0, scale: Optional[float] = None,
-                   qkv_bias: bool = True, out_bias: bool = False, out_scale: float = 1.0) -> PartSpec:
-    qw, kvw = heads_q * head_dim, heads_kv * head_dim
+                   qkv_bias: bool = True, out_bias: bool = False, out_scale: float = 1.0,
+                   v_dim: Optional[int] = None, qk_norm: bool = False, qk_norm_eps: float = 0.0,
+                   softcap: float = 0.0, sink: bool = False, value_mix: Optional[str] = None,
+                   value_mix_key: str = "values", names: Optional[dict] = None) -> PartSpec:
+    """``names``: what the file calls a role's tensor after ``prefix``, where that is not what
+    ``NAMES`` says."""
+    nm = dict(NAMES, **(names or {}))
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    qw, kw, vw = heads_q * head_dim, heads_kv * head_dim, heads_kv * v_dim
     tensors = {
-        "q_weight": TensorSpec(prefix + "q_proj.weight", (qw, width)),
-        "k_weight": TensorSpec(prefix + "k_proj.weight", (kvw, width)),
-        "v_weight": TensorSpec(prefix + "v_proj.weight", (kvw, width)),
-        "o_weight": TensorSpec(prefix + "o_proj.weight", (width, qw)),
+        "q_weight": TensorSpec(prefix + nm["q_weight"], (qw, width)),
+        "k_weight": TensorSpec(prefix + nm["k_weight"], (kw, width)),
+        "v_weight": TensorSpec(prefix + nm["v_weight"], (vw, width)),
+        "o_weight": TensorSpec(prefix + nm["o_weight"], (width, heads_q * v_dim)),
     }
     if qkv_bias:
-        tensors["q_bias"] = TensorSpec(prefix + "q_proj.bias", (qw,))
-        tensors["k_bias"] = TensorSpec(prefix + "k_proj.bias", (kvw,))
-        tensors["v_bias"] = TensorSpec(prefix + "v_proj.bias", (kvw,))
+        tensors["q_bias"] = TensorSpec(prefix + nm["q_bias"], (qw,))
+        tensors["k_bias"] = TensorSpec(prefix + nm["k_bias"], (kw,))
+        tensors["v_bias"] = TensorSpec(prefix + nm["v_bias"], (vw,))
     if out_bias:
-        tensors["o_bias"] = TensorSpec(prefix + "o_proj.bias", (width,))
+        tensors["o_bias"] = TensorSpec(prefix + nm["o_bias"], (width,))
+    if qk_norm:
+        tensors["q_norm"] = TensorSpec(prefix + nm["q_norm"], (head_dim,), init=(1.0, 0.02))
+        tensors["k_norm"] = TensorSpec(prefix + nm["k_norm"], (head_dim,), init=(1.0, 0.02))
+    if value_mix not in (None, "first", "mix"):
+        raise ValueError(f"value_mix is None, 'first' or 'mix', not {value_mix!r}")
+    if value_mix is not None:
+        # the first mixing layer's number is in the file too, and is not used
+        tensors["value_mix"] = TensorSpec(prefix + nm["value_mix"], (), init=(0.5, 0.1))
     return PartSpec("mixer", "attention", {
         "width": width, "heads_q": heads_q, "heads_kv": heads_kv, "head_dim": head_dim,
         "window": int(window), "scale": scale, "qkv_bias": qkv_bias, "out_bias": out_bias,
-        "out_scale": float(out_scale),
+        "out_scale": float(out_scale), "v_dim": v_dim, "qk_norm": bool(qk_norm), "qk_norm_eps": float(qk_norm_eps),
+        "softcap": float(softcap), "sink": bool(sink), "value_mix": value_mix, "value_mix_key": value_mix_key,
     }, tensors, {"position": position})
 
 
@@ -71,7 +99,26 @@ class Attention(Mixer):
         self.scale = float(np.float32(base_scale) * np.float32(self.position.score_scale))
         self.q_width = self.heads_q * self.head_dim
         self.kv_width = self.heads_kv * self.head_dim
-        if rt.fast_kernels:
+        self.v_dim = int(p.get("v_dim") or self.head_dim)
+        self.qk_norm = bool(p.get("qk_norm", False))
+        self.qk_norm_eps = float(p.get("qk_norm_eps", 0.0))
+        self.q_norm, self.k_norm = tensors.get("q_norm"), tensors.get("k_norm")
+        self.softcap = float(p.get("softcap", 0.0) or 0.0)
+        self.sink = bool(p.get("sink", False))
+        self.value_mix = p.get("value_mix")
+        self.value_mix_key = p.get("value_mix_key", "values")
+        self.lam = tensors.get("value_mix") if self.value_mix == "mix" else None
+        # head norms, capped scores, a sink, values of their own size or mixed values: the path whose
+        # kernels take them (no rotation there)
+        self.extended = bool(self.qk_norm or self.softcap or self.sink or self.value_mix or self.v_dim != self.head_dim)
+        if self.extended:
+            if self.position.rotary_tables() != (None, None, 0):
+                raise ValueError("head norms, capped scores, sinks and values of their own size are built for "
+                                 "mixers without a rotation")
+            if p.get("qkv_bias", True):
+                raise ValueError("head norms, capped scores, sinks and values of their own size are built for "
+                                 "mixers without biases on q, k and v")
+        if rt.fast_kernels and not self.extended:
             # (groups of one and two heads per kv head take higher tiles on the matrix cores)
             self.row_tile = ops.attention_row_tiles(self.heads_q, self.heads_kv, self.head_dim, rt.act_dtype)
 
@@ -101,7 +148,7 @@ class Attention(Mixer):
         self._q_parts = None
 
     def cache_spec(self) -> KVSpec:
-        return KVSpec(self.heads_kv, self.head_dim, self.window)
+        return KVSpec(self.heads_kv, self.head_dim, self.window, self.v_dim)
 
     fuses_norm = True
     graph_safe = True     # its launches depend on device buffers only
@@ -110,6 +157,48 @@ class Attention(Mixer):
     def forward(self, h, x, ctx, binding, then_norm=None):
         """x += attention(h).  Returns then_norm(x) when the output projection could apply the
         norm in its last pass, else None."""
+        a = self._attend(h, ctx, binding)
+        return self.out.add_into(a, x, then_norm, self.rt.act_dtype, scale=self.out_scale)
+
+    def produce(self, h, ctx, binding):
+        """attention(h) in float32 (whole, or in K slices of the output product), for a block that
+        adds it up itself."""
+        if self.out_scale != 1.0:
+            raise ValueError("a mixer that hands its result over has no multiplier of its own")
+        return self.out.raw(self._attend(h, ctx, binding))
+
+    def _attend_extended(self, h, ctx, binding):
+        rt = self.rt
+        writes = binding.writes_cache
+        if not writes:
+            self.query_only()
+        proj = self.qkv if writes else self._q_only
+        qkv = proj.partial(h)
+        if qkv is None:
+            qkv = proj(h, torch.float32)
+        v_first = v_out = None
+        if writes and self.value_mix is not None:
+            shared = ctx.shared
+            if self.value_mix == "first":
+                v_out = torch.empty((ctx.n_rows, self.heads_kv * self.v_dim), dtype=torch.float32, device=h.device)
+                shared[self.value_mix_key] = v_out
+            else:
+                v_first = shared.get(self.value_mix_key)
+                if v_first is None:
+                    raise RuntimeError(f"no earlier layer of this step has left its values under {self.value_mix_key!r}")
+        page_table = ctx.page_table(binding.group)
+        q = ops.headnorm_kv_store(qkv, rt.act_dtype, self.q_norm, self.k_norm, self.qk_norm_eps, ctx.row_pos, ctx.row_seq,
+                                  binding.k_cache, binding.v_cache, page_table, self.heads_q, self.heads_kv,
+                                  self.head_dim, self.v_dim, store=writes, v_first=v_first, lam=self.lam, v_out=v_out)
+        return ops.attention_capped(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
+                                    self.head_dim, self.v_dim, self.scale, self.window, self.softcap, self.sink,
+                                    fast=rt.fast_kernels)
+
+    def _attend(self, h, ctx, binding):
+        """The heads' results [rows, heads_q * v_dim] in the activation type; keys and values of the
+        step's rows are in the cache afterwards."""
+        if self.extended:
+            return self._attend_extended(h, ctx, binding)
         rt = self.rt
         writes = binding.writes_cache
         if not writes:
@@ -132,15 +221,13 @@ class Attention(Mixer):
                 qkv, rt.act_dtype, binding.k_cache.dtype, self.heads_q, self.heads_kv, self.head_dim,
                 rot_dims if inv_freq is not None else 0):
             # one token per sequence: rotation, store and attention in one kernel
-            a = ops.attention_decode_rope(qkv, inv_freq, freq_factors, rot_dims, binding.k_cache, binding.v_cache,
-                                          page_table, ctx.row_pos, self.heads_q, self.heads_kv, self.head_dim,
-                                          self.scale, self.window, bias=bias, store=writes)
-            return self.out.add_into(a, x, then_norm, rt.act_dtype, scale=self.out_scale)
+            return ops.attention_decode_rope(qkv, inv_freq, freq_factors, rot_dims, binding.k_cache, binding.v_cache,
+                                             page_table, ctx.row_pos, self.heads_q, self.heads_kv, self.head_dim,
+                                             self.scale, self.window, bias=bias, store=writes)
         q = ops.rope_kv_store(
             qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
             binding.k_cache if writes else None, binding.v_cache if writes else None,
             page_table if writes else None, self.heads_q, self.heads_kv if writes else 0, self.head_dim,
             bias=bias)
-        a = ops.attention(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
-                          self.head_dim, self.scale, self.window, fast=rt.fast_kernels, row_tile=self.row_tile)
-        return self.out.add_into(a, x, then_norm, rt.act_dtype, scale=self.out_scale)
+        return ops.attention(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
+                             self.head_dim, self.scale, self.window, fast=rt.fast_kernels, row_tile=self.row_tile)

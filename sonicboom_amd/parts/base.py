@@ -21,6 +21,9 @@ copy in the activation type, ``ctx`` the step's
                 takes ``then_norm=`` and may return the normed stream) and ``graph_safe``
                 (their launches depend on device buffers only, so a decode step may be
                 recorded once and replayed).
+                Mixers and feed-forwards may also offer ``produce(h, ctx[, binding])``, which returns the
+                result (a float32 tensor, K slices of it, or a :class:`Branch`) instead of adding it:
+                blocks that norm a sublayer's output need it.
 * **block**     ``mixer`` attribute and ``forward(x, ctx, binding, h=None, next_norm=None)``;
                 optionally ``first_norm``, the norm the block starts with (the block before
                 may then hand over ``h`` = first_norm(x) from its last pass), and calls of
@@ -57,13 +60,16 @@ class Runtime:
 @dataclass(frozen=True)
 class KVSpec:
     """What a mixer keeps per token: keys and values of ``kv_heads`` heads of
-    ``head_dim``; ``window`` > 0 when only the last ``window`` keys are read."""
+    ``head_dim``; ``window`` > 0 when only the last ``window`` keys are read; ``v_dim``: the
+    values' size per head when it is not the keys' (0: the same)."""
     kv_heads: int
     head_dim: int
     window: int = 0
+    v_dim: int = 0
 
     def key(self):
-        return (int(self.kv_heads), int(self.head_dim), int(self.window))
+        """(kv heads, head size, window, values' size)"""
+        return (int(self.kv_heads), int(self.head_dim), int(self.window), int(self.v_dim or self.head_dim))
 
 
 @dataclass(frozen=True)
@@ -84,6 +90,20 @@ class StateSpec:
     """Per-sequence state of fixed size (zeroed when a slot is handed out)."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class Branch:
+    """What a sublayer hands to a block that adds it up itself (``produce`` of mixers and
+    feed-forwards): the sum over s of a_s part_s (+ b extra).  ``part`` float32 [rows, width], or
+    slices [slices, rows, width], or with ``by_row`` [rows, slices, width]; ``part_weights``
+    float32 [rows, slices] (None: ones); ``extra`` float32 [rows, width] with ``extra_weights`` a
+    multiplier a row (None: one)."""
+    part: torch.Tensor
+    by_row: bool = False
+    part_weights: Optional[torch.Tensor] = None
+    extra: Optional[torch.Tensor] = None
+    extra_weights: Optional[torch.Tensor] = None
 
 
 class Part:

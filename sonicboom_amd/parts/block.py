@@ -6,10 +6,16 @@ feed-forward add their result into the float32 residual stream themselves,
 which lets their last projection fuse the addition (and a multiplier of the
 branch, the ``out_scale`` of their specs).  A block may have no feed-forward:
 it is then the first sublayer alone.
+
+``outnorm``: the sublayers read the stream as it is and the norm sits on what they give back:
+x += norm(mixer(x)); x += norm(ffn(x)).  The mixer and the feed-forward hand their result over
+(``produce``) and one pass sums its slices, norms it, adds it into the stream and leaves the new
+stream in the activation type for the sublayer that reads it next.
 """
 from __future__ import annotations
 
-from .base import Part, register_part
+from .. import ops
+from .base import Branch, Part, register_part
 from .spec import PartSpec
 
 
@@ -64,3 +70,71 @@ class PreNormBlock(Part):
         if trace is not None:
             trace("after_ffn", x)
         return out
+
+
+def outnorm_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec = None, ffn: PartSpec = None) -> PartSpec:
+    parts = {"mixer_norm": mixer_norm, "mixer": mixer}
+    if ffn is not None:
+        if ffn_norm is None:
+            raise ValueError("a block with a feed-forward needs the norm after it")
+        parts.update(ffn_norm=ffn_norm, ffn=ffn)
+    return PartSpec("block", "outnorm", {}, {}, parts)
+
+
+class StreamAsItIs:
+    """What a block that reads the stream itself names as its ``first_norm``: no norm, the stream
+    in the activation type.  A block before it that cannot produce that in its last pass is simply
+    followed by the conversion."""
+    fusable = False
+    weight = None
+
+    def forward(self, x, out_dtype, rows=None):
+        if rows is not None:
+            raise ValueError("the stream as it is has no picked rows")
+        return ops.cast(x, out_dtype)
+
+
+@register_part("block", "outnorm")
+class OutNormBlock(Part):
+    category = "block"
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        self.mixer_norm = parts["mixer_norm"]
+        self.first_norm = StreamAsItIs()
+        self.mixer = parts["mixer"]
+        self.ffn_norm = parts.get("ffn_norm")
+        self.ffn = parts.get("ffn")
+        for part, what in ((self.mixer, "mixer"), (self.ffn, "feed-forward")):
+            if part is not None and not hasattr(part, "produce"):
+                raise ValueError(f"a block that norms outputs needs a {what} that hands its result over (produce)")
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and (getattr(n, "groups", 1) != 1 or not hasattr(n, "eps")):
+                raise ValueError("a block that norms outputs takes RMS norms over whole rows")
+
+    def _join(self, x, y, norm, copy_dtype):
+        """x += norm(y); the new stream in ``copy_dtype`` (x itself when that is float32)."""
+        b = y if isinstance(y, Branch) else Branch(y)
+        return ops.norm_add(x, b.part, norm.weight, norm.eps, getattr(norm, "offset", 0.0), copy_dtype,
+                            part_weights=b.part_weights, extra=b.extra, extra_weights=b.extra_weights, by_row=b.by_row)
+
+    def forward(self, x, ctx, binding, h=None, next_norm=None):
+        """Run the block on the residual stream ``x`` in place.  ``h``: the stream in the activation
+        type when the block before has left it.  Returns the stream in the activation type when the
+        next block reads it as it is, else None."""
+        act = self.rt.act_dtype
+        if h is None:
+            h = ops.cast(x, act)
+        last = self.ffn is None
+        want = act if not last or isinstance(next_norm, StreamAsItIs) else None
+        h = self._join(x, self.mixer.produce(h, ctx, binding), self.mixer_norm, want)
+        trace = getattr(ctx, "trace", None)
+        if trace is not None:
+            trace("after_mixer", x)
+        if last:
+            return h
+        want = act if isinstance(next_norm, StreamAsItIs) else None
+        h = self._join(x, self.ffn.produce(h, ctx), self.ffn_norm, want)
+        if trace is not None:
+            trace("after_ffn", x)
+        return h

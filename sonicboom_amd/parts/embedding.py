@@ -20,10 +20,25 @@ def embedding_spec(name: str, vocab: int, width: int) -> PartSpec:
                     {"table": TensorSpec(name, (vocab, width))})
 
 
-def head_spec(name: str, vocab: int, width: int) -> PartSpec:
-    """``name`` may be the embedding table's name: the head then shares it."""
-    return PartSpec("head", "linear", {"vocab": vocab, "width": width},
+def head_spec(name: str, vocab: int, width: int, scale: float = 1.0) -> PartSpec:
+    """``name`` may be the embedding table's name: the head then shares it.  ``scale`` multiplies the logits."""
+    return PartSpec("head", "linear", {"vocab": vocab, "width": width, "scale": float(scale)},
                     {"weight": TensorSpec(name, (vocab, width))})
+
+
+def positional_embedding_spec(name: str, vocab: int, width: int, scale: float = 1.0, positions_name: str = None,
+                              n_positions: int = 0, norm_name: str = None, eps: float = 0.0,
+                              norm_offset: float = 0.0) -> PartSpec:
+    """x = table[id] * scale (+ positions[p], a learned row per position, not scaled), then, with
+    ``norm_name``, the RMS norm of that row times (norm_offset + weight)."""
+    tensors = {"table": TensorSpec(name, (vocab, width))}
+    if positions_name is not None:
+        tensors["positions"] = TensorSpec(positions_name, (n_positions, width))
+    if norm_name is not None:
+        tensors["norm_weight"] = TensorSpec(norm_name, (width,), init=(1.0 - float(norm_offset), 0.02))
+    return PartSpec("embedding", "positional", {"vocab": vocab, "width": width, "scale": float(scale),
+                                                "n_positions": int(n_positions), "eps": float(eps),
+                                                "norm_offset": float(norm_offset)}, tensors)
 
 
 @register_part("embedding", "lookup")
@@ -41,6 +56,28 @@ class Embedding(Part):
         return ops.embed(self.table, ids)
 
 
+@register_part("embedding", "positional")
+class PositionalEmbedding(Part):
+    """Token rows times a multiplier, plus a learned row per position, then optionally normed: one kernel."""
+    category = "embedding"
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        self.table = tensors["table"]
+        self.vocab, self.width = self.table.shape
+        self.positions = tensors.get("positions")
+        self.norm_weight = tensors.get("norm_weight")
+        p = spec.params
+        self.scale, self.eps, self.norm_offset = float(p.get("scale", 1.0)), float(p.get("eps", 0.0)), float(p.get("norm_offset", 0.0))
+        self.n_positions = self.positions.shape[0] if self.positions is not None else 0
+
+    def forward(self, ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        row_pos = ctx.row_pos if self.positions is not None else None
+        x, _ = ops.embed_pos_norm(self.table, ids, self.scale, self.positions, row_pos, self.norm_weight, self.eps,
+                                  self.norm_offset, norm=self.norm_weight is not None)
+        return x
+
+
 @register_part("head", "linear")
 class LinearHead(Part):
     category = "head"
@@ -49,6 +86,8 @@ class LinearHead(Part):
         super().__init__(spec, tensors, parts, rt)
         self.proj = Linear(tensors["weight"], None, rt.fast_kernels)
         self.vocab = int(spec.params["vocab"])
+        self.scale = float(spec.params.get("scale", 1.0))
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.proj(h, torch.float32)
+        logits = self.proj(h, torch.float32)
+        return logits if self.scale == 1.0 else ops.scale_(logits, self.scale)

@@ -4,7 +4,7 @@
 
 /root/reference/core/src/model/emit.cpp:364-374; the activation is a parameter
 of the spec: "silu", g / (1 + exp(-g)) (/root/reference/core/src/nn/activation.cpp:41-50),
-or "gelu_tanh", 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))) (:27-36); the product
+"gelu_tanh", 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))) (:27-36), or "relu", max(g, 0); the product
 kernels apply either in their epilogue.  The gate and up matrices
 are stacked into one [2*inner, width] matrix when the part is built, so a
 step runs one product for both; its float32 result feeds the activation
@@ -26,15 +26,17 @@ from .base import Part, register_part
 from .linear import Linear
 from .spec import PartSpec, TensorSpec
 
-ACTIVATIONS = ("silu", "gelu_tanh")    # the gates the product kernels apply in their epilogue
+ACTIVATIONS = ("silu", "gelu_tanh", "relu")    # the gates the product kernels apply in their epilogue
 
 
-def gated_ffn_spec(prefix: str, width: int, inner: int, activation: str = "silu", out_scale: float = 1.0) -> PartSpec:
+def gated_ffn_spec(prefix: str, width: int, inner: int, activation: str = "silu", out_scale: float = 1.0,
+                   names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")) -> PartSpec:
+    """``names``: what the file calls the gate, up and down matrices after ``prefix``."""
     return PartSpec("ffn", "gated_dense", {"width": width, "inner": inner, "activation": activation,
                                            "out_scale": float(out_scale)}, {
-        "gate_weight": TensorSpec(prefix + "gate_proj.weight", (inner, width)),
-        "up_weight": TensorSpec(prefix + "up_proj.weight", (inner, width)),
-        "down_weight": TensorSpec(prefix + "down_proj.weight", (width, inner)),
+        "gate_weight": TensorSpec(prefix + names[0], (inner, width)),
+        "up_weight": TensorSpec(prefix + names[1], (inner, width)),
+        "down_weight": TensorSpec(prefix + names[2], (width, inner)),
     })
 
 
@@ -65,6 +67,12 @@ class GatedDenseFFN(Part):
         norm in its last pass, else None."""
         mid = self.gate_up.gated_product(h, self.rt.act_dtype)
         return self.down.add_into(mid, x, then_norm, self.rt.act_dtype, scale=self.out_scale)
+
+    def produce(self, h, ctx):
+        """ffn(h) in float32 (whole, or in K slices), for a block that adds it up itself."""
+        if self.out_scale != 1.0:
+            raise ValueError("a feed-forward that hands its result over has no multiplier of its own")
+        return self.down.raw(self.gate_up.gated_product(h, self.rt.act_dtype))
 
 
 def dense_ffn_spec(up_name: str, down_name: str, width: int, inner: int, activation: str,

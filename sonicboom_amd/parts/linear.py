@@ -72,6 +72,12 @@ class Linear:
             return None
         return ops.gemm_bf16_partial(x, self.packed, packed_shape=(self.rows, self.n_in))
 
+    def raw(self, x: torch.Tensor) -> torch.Tensor:
+        """The product in float32 for a consumer that adds it up itself: [slices, rows, out] when a
+        kernel that cuts K over the grid takes the call (no bias then), else [rows, out]."""
+        part = self.partial(x) if self.bias is None else None
+        return part if part is not None else self(x, torch.float32)
+
     def add_into(self, x: torch.Tensor, resid: torch.Tensor, then_norm=None, out_dtype=None, scale: float = 1.0):
         """resid += scale * (x W^T (+ b)).  With ``then_norm`` (an RMS norm part, whole rows or in
         groups) tries to return then_norm(resid) in ``out_dtype`` from the same pass; None when the

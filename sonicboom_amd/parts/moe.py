@@ -1,0 +1,114 @@
+"""A feed-forward of routed experts.
+
+    z = W_router f;   the ``top`` largest z are chosen (ties to the lower number), their weights
+    are the softmax over the chosen z alone;   y = sum over the chosen e of weight_e expert_e(f)
+    (+ sigmoid(w_sg . f) shared(f), an expert that every row takes, when the spec has one)
+
+    expert(f) = W_down (g' sigmoid(alpha g') (u' + 1)),  g' = min(W_gate f, limit),
+    u' = W_up f cut to [-limit, limit]                                  ("swish_clamp")
+
+The router runs in float32 whatever the model's type (its matrix, with the shared expert's gate
+row under it, is kept in float32 and takes the plain product).  Choice and weights are made on the
+device, and the experts' products find their rows there too: nothing of a step depends on a value the
+host has seen, so a decode step can be recorded and replayed.  The experts' matrices are stacked
+when the part is built: [experts, 2 * inner, width] (gate over up) and [experts, width, inner].
+
+Every (row, choice) pair has its own row of the intermediate and of the result; the pass that
+ends the sublayer adds a row's pairs in the order of the choice, times their weights.  A pair's
+numbers depend on its row and its expert alone, never on which other rows chose the same expert.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import Branch, Part, register_part
+from .linear import Linear
+from .spec import PartSpec, TensorSpec
+
+EXPERT_ACTIVATIONS = ("swish_clamp",)
+
+
+def moe_ffn_spec(prefix: str, width: int, experts: int, top: int, inner: int, limit: float, alpha: float = 1.702,
+                 shared_inner: int = 0, shared_limit: float = 0.0, activation: str = "swish_clamp",
+                 names=("gate", "up", "down"), expert_prefix: str = "e{}.", router_name: str = "router",
+                 shared_prefix: str = "shared.", shared_gate_name: str = "shared.sg") -> PartSpec:
+    """``shared_inner`` > 0: an expert of that inner width that every row takes, times the sigmoid of
+    one more router row (``shared_gate_name``)."""
+    tensors = {"router": TensorSpec(prefix + router_name, (experts, width))}
+    for e in range(experts):
+        ep = prefix + expert_prefix.format(e)
+        tensors[f"e{e}.gate"] = TensorSpec(ep + names[0], (inner, width))
+        tensors[f"e{e}.up"] = TensorSpec(ep + names[1], (inner, width))
+        tensors[f"e{e}.down"] = TensorSpec(ep + names[2], (width, inner))
+    if shared_inner:
+        sp = prefix + shared_prefix
+        tensors["shared.gate"] = TensorSpec(sp + names[0], (shared_inner, width))
+        tensors["shared.up"] = TensorSpec(sp + names[1], (shared_inner, width))
+        tensors["shared.down"] = TensorSpec(sp + names[2], (width, shared_inner))
+        tensors["shared.sg"] = TensorSpec(prefix + shared_gate_name, (1, width))
+    return PartSpec("ffn", "moe", {"width": width, "experts": experts, "top": top, "inner": inner, "limit": float(limit),
+                                   "alpha": float(alpha), "shared_inner": int(shared_inner),
+                                   "shared_limit": float(shared_limit), "activation": activation}, tensors)
+
+
+def _stack(mats):
+    if any(m.dtype != mats[0].dtype for m in mats):
+        mats = [m.float() for m in mats]
+    return torch.stack(mats, dim=0).contiguous()
+
+
+@register_part("ffn", "moe")
+class MoEFFN(Part):
+    category = "ffn"
+    graph_safe = True     # its launches depend on device buffers only
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        p = spec.params
+        self.width, self.experts, self.top, self.inner = int(p["width"]), int(p["experts"]), int(p["top"]), int(p["inner"])
+        self.limit, self.alpha = float(p["limit"]), float(p.get("alpha", 1.702))
+        self.shared_inner, self.shared_limit = int(p.get("shared_inner", 0)), float(p.get("shared_limit", 0.0))
+        if p.get("activation", "swish_clamp") not in EXPERT_ACTIVATIONS:
+            raise ValueError(f"unknown expert activation {p.get('activation')!r}; known: {EXPERT_ACTIVATIONS}")
+        if not 0 < self.top <= self.experts:
+            raise ValueError(f"{self.top} choices of {self.experts} experts")
+        if self.top > ops.MOE_MAX_TOP:
+            raise ValueError(f"{self.top} choices a row are more than the router kernel's {ops.MOE_MAX_TOP}")
+        rows = [tensors["router"].float()]
+        if self.shared_inner:
+            rows.append(tensors["shared.sg"].float().reshape(1, self.width))
+        self.router = Linear(torch.cat(rows, dim=0), None, rt.fast_kernels)          # float32: the plain product
+        self.w_in = ops.MoEWeight(_stack([torch.cat([tensors[f"e{e}.gate"], tensors[f"e{e}.up"]], dim=0)
+                                          for e in range(self.experts)]), gated=True, fast=rt.fast_kernels)
+        self.w_out = ops.MoEWeight(_stack([tensors[f"e{e}.down"] for e in range(self.experts)]), fast=rt.fast_kernels)
+        self.s_in = self.s_out = None
+        if self.shared_inner:
+            self.s_in = ops.MoEWeight(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0).unsqueeze(0).contiguous(),
+                                      gated=True, fast=rt.fast_kernels)
+            self.s_out = ops.MoEWeight(tensors["shared.down"].unsqueeze(0).contiguous(), fast=rt.fast_kernels)
+
+    def produce(self, h, ctx):
+        """The pairs' results [rows, top, width] with their weights, and the shared expert's with its
+        gate, for the pass that adds them up."""
+        act = self.rt.act_dtype
+        n = h.shape[0]
+        z = self.router(h, torch.float32)                                  # [n, experts (+ 1)]
+        ids, weights = ops.moe_route(z, self.experts, self.top, has_gate=bool(self.shared_inner))
+        plan = ops.moe_plan(ids, self.experts)
+        mid = ops.moe_product(h, self.w_in, plan, self.top, act, self.limit, self.alpha)       # [n * top, inner]
+        out = ops.moe_product(mid, self.w_out, plan, 1, torch.float32)                         # [n * top, width]
+        branch = Branch(out.view(n, self.top, self.width), by_row=True, part_weights=weights[:, : self.top])
+        if self.shared_inner:
+            every = ops.moe_plan(None, 1, n_pairs=n, device=h.device)
+            smid = ops.moe_product(h, self.s_in, every, 1, act, self.shared_limit, self.alpha)
+            branch.extra = ops.moe_product(smid, self.s_out, every, 1, torch.float32)
+            branch.extra_weights = weights[:, self.top:]
+        return branch
+
+    def forward(self, h, x, ctx, then_norm=None):
+        """x += moe(h)."""
+        b = self.produce(h, ctx)
+        ops.norm_add(x, b.part, None, 0.0, 0.0, None, part_weights=b.part_weights, extra=b.extra,
+                     extra_weights=b.extra_weights, by_row=True, norm=False)
+        return None

@@ -127,7 +127,8 @@ def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
 
 
 def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
-    return (b.astype(np.uint32) << 16).view(np.float32)
+    b = np.asarray(b)
+    return (b.astype(np.uint32).reshape(-1) << 16).view(np.float32).reshape(b.shape)      # also a tensor of no axes
 
 
 def write_safetensors(path: str, tensors: Iterable[Tuple[str, str, np.ndarray]], metadata=None) -> None:
