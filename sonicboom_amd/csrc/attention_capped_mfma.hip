@@ -1,0 +1,293 @@
+// Attention on the matrix cores for mixers whose keys and values have sizes of their own, whose
+// scores may be capped by a tanh and whose softmax may hold a sink (one more key of score 0
+// without a value): compiled with -DSB_KEY_DIM=<dk> -DSB_VALUE_DIM=<dv>, both multiples of 16.
+//
+// One kernel for prompt steps and single rows.  A block is a run of up to 16 consecutive rows of
+// one sequence (a row tile) times one kv head; its four waves are four query heads of that kv
+// head's group (more heads: further blocks).  Every page of the cache is staged once per block in
+// LDS as it lies (the cache keeps a page's rows in the order the fragments are read without bank
+// conflicts: sb_key_index, sb_value_index) and shared by the waves; the next page's loads are in
+// flight while this one is attended.
+//
+//   S^T = K Q^T   MFMA 16x16x32, A = 16 keys x 32 d from LDS, B = Q^T kept in registers
+//   O^T = V^T P^T MFMA 16x16x32, A = 16 d x 32 keys from LDS, B = P^T straight from the S^T tiles:
+//         row r of an S^T tile stands for key 8 (r / 4) + 4 t + r % 4 of a half page (t the tile), so
+//         the eight probabilities a lane holds after two tiles are eight consecutive keys.
+//
+// Softmax in float32, running maximum and sum per query column; a sink starts the maximum at 0 and
+// the sum at 1.  Steps of few rows share the pages of a sequence out over `chunks` blocks, which
+// leave (unnormed result, maximum, sum) for sb_cattn_merge.
+#include "mfma.h"
+
+#if !defined(SB_KEY_DIM) || !defined(SB_VALUE_DIM)
+#error "compile with -DSB_KEY_DIM=<key size> -DSB_VALUE_DIM=<value size>"
+#endif
+static_assert(SB_KEY_DIM % 16 == 0 && SB_KEY_DIM >= 16 && SB_KEY_DIM <= 256, "key size: 16..256 in steps of 16");
+static_assert(SB_VALUE_DIM % 16 == 0 && SB_VALUE_DIM >= 16 && SB_VALUE_DIM <= 256, "value size: 16..256 in steps of 16");
+
+namespace sb {
+char *error_slot() {
+  static thread_local char slot[kErrorLen] = "";
+  return slot;
+}
+}  // namespace sb
+
+extern "C" const char *sb_cattn_last_error(void) { return sb::error_slot(); }
+extern "C" int sb_cattn_key_dim(void) { return SB_KEY_DIM; }
+extern "C" int sb_cattn_value_dim(void) { return SB_VALUE_DIM; }
+
+namespace {
+
+constexpr int DK = SB_KEY_DIM, DV = SB_VALUE_DIM;
+constexpr int KSTEPS = (DK + 31) / 32;      // steps of 32 d of the score product
+constexpr int DT = DV / 16;                 // tiles of 16 d of the result
+constexpr int NW = 4;                       // waves (query heads) a block
+constexpr int kThreads = 64 * NW;
+constexpr int kKeyChunks = SB_PAGE * DK / 8;    // 16-byte chunks of a page's keys of one head
+constexpr int kValChunks = SB_PAGE * DV / 8;
+constexpr int kKeyLoads = (kKeyChunks + kThreads - 1) / kThreads;
+constexpr int kValLoads = (kValChunks + kThreads - 1) / kThreads;
+constexpr int kTile = 16;
+
+struct Args {
+  bf16_t *out;                 // [rows, heads_q * DV], or NULL when partial results are written
+  float *part_o, *part_ml;     // [chunks][rows][heads_q][DV], [chunks][rows][heads_q][2]
+  const bf16_t *q;             // [rows, heads_q * DK]
+  const bf16_t *k_cache, *v_cache;
+  const int32_t *page_table; int max_pages, n_pages;
+  const int32_t *row_pos, *tiles;
+  int n_rows, heads_q, heads_kv;
+  float scale, softcap; int window, sink, chunk_pages;
+};
+
+// softcap * tanh(s / softcap) with the fast exponential: tanh(x) = 1 - 2 / (exp(2x) + 1)
+__device__ __forceinline__ float capped(float s, float cap, float inv_cap) {
+  const float x = fminf(fmaxf(s * inv_cap, -15.0f), 15.0f);
+  return cap * (1.0f - 2.0f / (__expf(2.0f * x) + 1.0f));
+}
+
+__global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
+  __shared__ uint4 k_lds[kKeyChunks];
+  __shared__ uint4 v_lds[kValChunks];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
+  const int group = a.heads_q / a.heads_kv, zgroups = (group + NW - 1) / NW;
+  const int kvh = blockIdx.y / zgroups, hz = blockIdx.y % zgroups;
+  const int hg = hz * NW + wave;                  // the wave's head within the group
+  const bool has_head = hg < group;
+  const int h = kvh * group + (has_head ? hg : 0);
+  const int32_t *tile = a.tiles + size_t(blockIdx.x) * 4;
+  const int r0 = tile[0], nr = tile[1], seq = tile[2];
+  const int chunk = blockIdx.z;
+  const int p0 = a.row_pos[r0], p_last = p0 + nr - 1;
+  const int lo = (a.window > 0 && p0 >= a.window) ? p0 - a.window + 1 : 0;      // oldest key any row of the tile reads
+  int page_lo = lo / SB_PAGE, page_hi = p_last / SB_PAGE;
+  if (a.chunk_pages > 0) {
+    page_lo = max(page_lo, chunk * a.chunk_pages);
+    page_hi = min(page_hi, (chunk + 1) * a.chunk_pages - 1);
+  }
+  const int32_t *table = a.page_table + size_t(seq) * a.max_pages;
+
+  // the queries of the wave's head: B operand, column = row of the tile
+  bf16x8_t qf[KSTEPS];
+#pragma unroll
+  for (int kc = 0; kc < KSTEPS; ++kc) {
+    const int d = 32 * kc + 8 * g;
+    qf[kc] = as_bf16x8(ld16(a.q + (size_t(r0 + col) * a.heads_q + h) * DK + d, has_head && col < nr && d < DK));
+  }
+  const int q_pos = p0 + col;
+  const int q_lo = (a.window > 0 && q_pos >= a.window) ? q_pos - a.window + 1 : 0;
+
+  const float neg_inf = -__builtin_inff();
+  const bool with_sink = a.sink && chunk == 0;
+  float m = with_sink ? 0.0f : neg_inf;
+  float l = (with_sink && g == 0) ? 1.0f : 0.0f;      // a lane's share of the column's sum
+  floatx4_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  const float inv_cap = a.softcap > 0.0f ? 1.0f / a.softcap : 0.0f;
+
+  uint4 kreg[kKeyLoads], vreg[kValLoads];
+  auto fetch = [&](int c) {
+    int page = (c >= 0 && c < a.max_pages) ? table[c] : -1;
+    if (page >= a.n_pages) page = -1;
+    const uint4 *kp = reinterpret_cast<const uint4 *>(a.k_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DK);
+    const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DV);
+#pragma unroll
+    for (int i = 0; i < kKeyLoads; ++i) {
+      const int idx = tid + i * kThreads;
+      kreg[i] = (page >= 0 && idx < kKeyChunks) ? kp[idx] : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int i = 0; i < kValLoads; ++i) {
+      const int idx = tid + i * kThreads;
+      vreg[i] = (page >= 0 && idx < kValChunks) ? vp[idx] : make_uint4(0u, 0u, 0u, 0u);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < kKeyLoads; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < kKeyChunks) k_lds[idx] = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kValLoads; ++i) {
+      const int idx = tid + i * kThreads;
+      if (idx < kValChunks) v_lds[idx] = vreg[i];
+    }
+  };
+
+  if (page_lo <= page_hi) fetch(page_lo);
+  for (int c = page_lo; c <= page_hi; ++c) {
+    __syncthreads();            // the page before has been read by every wave
+    stage();
+    __syncthreads();
+    if (c < page_hi) fetch(c + 1);
+    if (!has_head) continue;
+    const bf16_t *kl = reinterpret_cast<const bf16_t *>(k_lds);
+    const bf16_t *vl = reinterpret_cast<const bf16_t *>(v_lds);
+#pragma unroll
+    for (int hp = 0; hp < 2; ++hp) {
+      const int first = c * SB_PAGE + 32 * hp;          // position of the half page's first key
+      if (first > p_last || first + 31 < lo) continue;  // uniform over the block
+      floatx4_t s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        const int slot = 32 * hp + 8 * (col >> 2) + 4 * t + (col & 3);
+#pragma unroll
+        for (int kc = 0; kc < KSTEPS; ++kc) {
+          const int d = 32 * kc + 8 * g;
+          uint4 kf = make_uint4(0u, 0u, 0u, 0u);
+          if (d < DK) kf = *reinterpret_cast<const uint4 *>(kl + sb_key_index(slot, d, DK));
+          s[t] = mfma16(as_bf16x8(kf), qf[kc], s[t]);
+        }
+      }
+      // the lane's eight scores: keys first + 8 g + 4 t + i of query column `col`
+      float sc[8];
+      float mx = neg_inf;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = first + 8 * g + 4 * t + i;
+          float v = s[t][i] * a.scale;
+          if (a.softcap > 0.0f) v = capped(v, a.softcap, inv_cap);
+          const bool visible = col < nr && j <= q_pos && j >= q_lo;
+          v = visible ? v : neg_inf;
+          sc[4 * t + i] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = max_over_lane_groups(mx);
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m == neg_inf ? 0.0f : __expf(m - m_new);
+      float psum = 0.0f, p[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = sc[e] == neg_inf ? 0.0f : __expf(sc[e] - m_new);
+        psum += p[e];
+      }
+      l = l * alpha + psum;
+      m = m_new;
+      uint4 pw;
+      pw.x = pack_bf16(p[0], p[1]); pw.y = pack_bf16(p[2], p[3]);
+      pw.z = pack_bf16(p[4], p[5]); pw.w = pack_bf16(p[6], p[7]);
+      const bf16x8_t pf = as_bf16x8(pw);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int d = 16 * dt + col;
+        const uint4 vf = *reinterpret_cast<const uint4 *>(vl + sb_value_index(d, 32 * hp + 8 * g));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
+        o[dt] = mfma16(as_bf16x8(vf), pf, o[dt]);
+      }
+    }
+  }
+
+  // the column's sum over the four lane groups
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!has_head || col >= nr) return;
+  const int row = r0 + col;
+  if (a.out) {
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    bf16_t *dst = a.out + (size_t(row) * a.heads_q + h) * DV;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 w;
+      w.x = pack_bf16(o[dt][0] * inv, o[dt][1] * inv);
+      w.y = pack_bf16(o[dt][2] * inv, o[dt][3] * inv);
+      *reinterpret_cast<uint2 *>(dst + 16 * dt + 4 * g) = w;
+    }
+  } else {
+    const size_t at = (size_t(chunk) * a.n_rows + row) * a.heads_q + h;
+    float *dst = a.part_o + at * DV;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<float4 *>(dst + 16 * dt + 4 * g) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
+    if (g == 0) {
+      a.part_ml[at * 2] = m;
+      a.part_ml[at * 2 + 1] = l;
+    }
+  }
+}
+
+// out[row][h][:] = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M), M the largest m_c: a thread a number
+__global__ void __launch_bounds__(256)
+merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml, int chunks,
+             size_t n_heads /* rows * heads_q */) {
+  const size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= n_heads * DV) return;
+  const size_t rh = idx / DV;
+  float big = -__builtin_inff();
+  for (int c = 0; c < chunks; ++c) big = fmaxf(big, part_ml[(size_t(c) * n_heads + rh) * 2]);
+  float num = 0.0f, den = 0.0f;
+  for (int c = 0; c < chunks; ++c) {
+    const float mc = part_ml[(size_t(c) * n_heads + rh) * 2];
+    if (mc == -__builtin_inff()) continue;
+    const float w = __expf(mc - big);
+    num = fmaf(w, part_o[size_t(c) * n_heads * DV + idx], num);
+    den = fmaf(w, part_ml[(size_t(c) * n_heads + rh) * 2 + 1], den);
+  }
+  out[idx] = f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+}
+
+}  // namespace
+
+extern "C" int sb_cattn_tile_rows(void) { return kTile; }
+
+// out bf16 [rows, heads_q * dv]; q bf16 [rows, heads_q * dk]; tiles int32 [n_tiles, 4] = (first row,
+// rows <= 16, sequence, 0), consecutive rows of one sequence.  chunks > 1: the pages of every tile
+// are shared out over that many blocks of chunk_pages pages each (chunks * chunk_pages >= max_pages)
+// and merged; part_o f32 [chunks * rows * heads_q * dv] and part_ml f32 [chunks * rows * heads_q * 2]
+// are the scratch for that.
+extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                             const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
+                             const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
+                             int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
+                             float *part_ml, void *stream) {
+  SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && tiles, "sb_cattn_bf16: null pointer");
+  SB_REQUIRE(n_tiles >= 0 && n_rows >= 0 && heads_q > 0 && heads_kv > 0 && max_pages > 0 && n_pages > 0 && window >= 0,
+             "sb_cattn_bf16: bad sizes tiles=%d rows=%d heads=%d/%d", n_tiles, n_rows, heads_q, heads_kv);
+  SB_REQUIRE(heads_q % heads_kv == 0, "sb_cattn_bf16: %d query heads are not a multiple of %d kv heads", heads_q, heads_kv);
+  SB_REQUIRE(softcap >= 0.0f, "sb_cattn_bf16: the cap of the scores must not be negative");
+  SB_REQUIRE(chunks >= 1 && (chunks == 1 || (part_o && part_ml && chunk_pages > 0 &&
+                                             (long long)chunks * chunk_pages >= max_pages)),
+             "sb_cattn_bf16: %d chunks of %d pages do not cover %d pages, or have no scratch", chunks, chunk_pages, max_pages);
+  if (n_tiles == 0 || n_rows == 0) return SB_OK;
+  const int group = heads_q / heads_kv, zgroups = (group + NW - 1) / NW;
+  SB_SUPPORT((long long)heads_kv * zgroups <= 65535 && chunks <= 65535, "sb_cattn_bf16: too many heads or chunks for one grid");
+  hipStream_t s = (hipStream_t)stream;
+  Args a;
+  a.out = chunks == 1 ? (bf16_t *)out : nullptr;
+  a.part_o = part_o; a.part_ml = part_ml;
+  a.q = (const bf16_t *)q; a.k_cache = (const bf16_t *)k_cache; a.v_cache = (const bf16_t *)v_cache;
+  a.page_table = page_table; a.max_pages = max_pages; a.n_pages = n_pages; a.row_pos = row_pos; a.tiles = tiles;
+  a.n_rows = n_rows; a.heads_q = heads_q; a.heads_kv = heads_kv; a.scale = scale; a.softcap = softcap;
+  a.window = window; a.sink = sink; a.chunk_pages = chunks == 1 ? 0 : chunk_pages;
+  capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups, chunks), kThreads, 0, s>>>(a);
+  int st = sb::check_launch("sb_cattn_bf16");
+  if (st != SB_OK || chunks == 1) return st;
+  const size_t n = size_t(n_rows) * heads_q * DV;
+  merge_kernel<<<unsigned((n + 255) / 256), 256, 0, s>>>((bf16_t *)out, part_o, part_ml, chunks, size_t(n_rows) * heads_q);
+  return sb::check_launch("sb_cattn_merge");
+}

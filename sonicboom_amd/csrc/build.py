@@ -5,7 +5,9 @@ Two kinds of library come out of it:
 * ``libsbhip.so`` — every kernel whose code does not depend on the model;
 * ``libsbattn_hd<N>.so`` — the MFMA attention kernels for one head size N,
   compiled when a model of that head size is first built (or ahead of time by
-  :func:`build_all`).
+  :func:`build_all`);
+* ``libsbcattn_k<K>_v<V>.so`` — the MFMA kernels of attention with capped scores and a
+  sink for keys of K and values of V numbers a head, compiled the same way.
 
 A library lives in ``_build/`` beside the sources together with a stamp that
 holds the hash of the sources and flags it was made from.  :func:`ensure`
@@ -44,6 +46,9 @@ CORE_SOURCES = [
 ]
 HEADERS = ["common.h", "sb_hip.h", "mfma.h"]
 ATTN_SOURCES = ["attention_mfma.hip"]
+CAPPED_ATTN_SOURCES = ["attention_capped_mfma.hip"]
+# (key size, value size) pairs of the capped attention kernels compiled ahead of time by build_all()
+PREBUILT_CAPPED_DIMS = ((64, 64), (128, 128), (128, 64), (192, 128), (32, 16), (48, 32), (16, 48))
 
 # Head sizes compiled ahead of time by build_all(): every size the kernels take.
 PREBUILT_HEAD_DIMS = tuple(range(16, 257, 16))
@@ -182,6 +187,17 @@ def ensure_attention(head_dim: int, force: bool = False) -> str:
     return _ensure(f"libsbattn_hd{head_dim}.so", ATTN_SOURCES, [f"SB_HEAD_DIM={head_dim}"], force)
 
 
+def ensure_capped_attention(key_dim: int, value_dim: int, force: bool = False) -> str:
+    """Path of the MFMA library of attention with capped scores and a sink for one pair of key and
+    value sizes."""
+    for n in (key_dim, value_dim):
+        if n % 16 or not 16 <= n <= MAX_HEAD_DIM:
+            raise BuildError(f"the capped attention kernels take key and value sizes 16..{MAX_HEAD_DIM} in steps of 16, "
+                             f"not {key_dim} and {value_dim}")
+    return _ensure(f"libsbcattn_k{key_dim}_v{value_dim}.so", CAPPED_ATTN_SOURCES,
+                   [f"SB_KEY_DIM={key_dim}", f"SB_VALUE_DIM={value_dim}"], force)
+
+
 def ensure_plain_host(force: bool = False) -> str:
     """Path of ``libsbplain.so``: the kernels' plain C++ twins on host memory (plain_host.cpp),
     compiled with the host compiler.  The tests compare the kernels with them."""
@@ -219,6 +235,9 @@ def build_all(force: bool = True) -> None:
     if _existing(ATTN_SOURCES):
         with ThreadPoolExecutor(max_workers=_jobs()) as ex:
             list(ex.map(lambda hd: ensure_attention(hd, force=force), PREBUILT_HEAD_DIMS))
+    if _existing(CAPPED_ATTN_SOURCES):
+        with ThreadPoolExecutor(max_workers=_jobs()) as ex:
+            list(ex.map(lambda kv: ensure_capped_attention(*kv, force=force), PREBUILT_CAPPED_DIMS))
 
 
 if __name__ == "__main__":

@@ -1281,9 +1281,61 @@ def attention_capped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      heads_q: int, heads_kv: int, head_dim: int, v_dim: int, scale: float, window: int,
                      softcap: float, sink: bool, fast: bool = True) -> torch.Tensor:
     """Attention of a step's rows over the cache with values of their own size, capped scores and a
-    sink (see :func:`attention_capped_plain`)."""
+    sink (see :func:`attention_capped_plain`).  bfloat16 with key and value sizes in steps of 16
+    runs on the matrix cores; everything else takes the plain kernel."""
+    if fast and capped_attention_mfma_ok(q.dtype, k_cache.dtype, head_dim, v_dim):
+        return attention_capped_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(CAPPED_ROW_TILE),
+                                     heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink)
     return attention_capped_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                                   head_dim, v_dim, scale, window, softcap, sink)
+
+
+CAPPED_ROW_TILE = 16        # rows of a run that a block of the matrix-core kernel takes (sb_cattn_tile_rows)
+CAPPED_SPLIT_BLOCKS = 512   # blocks a step of few rows aims at by sharing out its pages
+
+
+def capped_attention_mfma_ok(q_dtype, cache_dtype, head_dim: int, v_dim: int) -> bool:
+    return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16
+            and all(n % 16 == 0 and 16 <= n <= MFMA_MAX_HEAD_DIM for n in (head_dim, v_dim)))
+
+
+def attention_capped_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                          row_pos: torch.Tensor, tiles: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
+                          v_dim: int, scale: float, window: int, softcap: float, sink: bool,
+                          chunks: Optional[int] = None) -> torch.Tensor:
+    """The matrix-core form of :func:`attention_capped_plain`.  ``tiles`` int32 [n, 4]: the rows in
+    runs of up to 16 consecutive rows of one sequence.  ``chunks``: over how many blocks a run's
+    pages are shared out (None: chosen from the shapes alone, so that a recorded step replays)."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, tiles)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
+        raise KernelLibraryError(f"queries must be bfloat16 [rows, {heads_q * head_dim}]")
+    _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
+    if k_cache.dtype != torch.bfloat16:
+        raise KernelLibraryError("the matrix-core kernel reads a bfloat16 cache")
+    _i32(row_pos, n, "row positions")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+    if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 4:
+        raise KernelLibraryError("row tiles must be int32 [n, 4]")
+    n_tiles, max_pages = tiles.shape[0], page_table.shape[1]
+    group = heads_q // heads_kv
+    blocks = max(1, n_tiles * heads_kv * ((group + 3) // 4))
+    if chunks is None:
+        chunks = max(1, min(max_pages, CAPPED_SPLIT_BLOCKS // blocks))
+    chunk_pages = (max_pages + chunks - 1) // chunks
+    chunks = (max_pages + chunk_pages - 1) // chunk_pages
+    part_o = part_ml = None
+    if chunks > 1:
+        part_o = torch.empty((chunks, n, heads_q, v_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((chunks, n, heads_q, 2), dtype=torch.float32, device=q.device)
+    out = torch.empty((n, heads_q * v_dim), dtype=torch.bfloat16, device=q.device)
+    lib = library.capped_attention_library(head_dim, v_dim)
+    check(lib.sb_cattn_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages, k_cache.shape[0],
+                            _p(row_pos), _p(tiles), n_tiles, n, heads_q, heads_kv, float(scale), int(window),
+                            float(softcap), 1 if sink else 0, chunks, chunk_pages, _p(part_o), _p(part_ml), _stream()),
+          lib, "sb_cattn_last_error")
+    return out
 
 
 def moe_max_top() -> int:

@@ -96,9 +96,19 @@ _ATTN_SIGNATURES = {
     "sb_attn_head_dim": [],
 }
 
+_CAPPED_ATTN_SIGNATURES = {
+    # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, n_rows, heads_q, heads_kv,
+    # scale, window, softcap, sink, chunks, chunk_pages, part_o, part_ml, stream
+    "sb_cattn_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P],
+    "sb_cattn_tile_rows": [],
+    "sb_cattn_key_dim": [],
+    "sb_cattn_value_dim": [],
+}
+
 _lock = threading.Lock()
 _core = None
 _attn = {}
+_cattn = {}
 
 
 def _declare(lib, table, optional=False):
@@ -161,12 +171,33 @@ def attention_library(head_dim: int):
     return lib
 
 
+def capped_attention_library(key_dim: int, value_dim: int):
+    """The MFMA library of attention with capped scores and a sink for one pair of sizes, built on first use."""
+    key = (int(key_dim), int(value_dim))
+    lib = _cattn.get(key)
+    if lib is None:
+        with _lock:
+            lib = _cattn.get(key)
+            if lib is None:
+                try:
+                    path = build.ensure_capped_attention(*key)
+                    lib = ctypes.CDLL(path)
+                except (build.BuildError, OSError) as e:
+                    raise KernelLibraryError(f"cannot load the capped attention kernels for sizes {key}: {e}") from e
+                lib.sb_cattn_last_error.restype = c_char_p
+                _declare(lib, _CAPPED_ATTN_SIGNATURES)
+                lib._sb_path = path
+                _cattn[key] = lib
+    return lib
+
+
 def loaded_paths():
     """Paths of the shared libraries this process has loaded."""
     out = []
     if _core is not None:
         out.append(_core._sb_path)
     out += [lib._sb_path for lib in _attn.values()]
+    out += [lib._sb_path for lib in _cattn.values()]
     return out
 
 

@@ -164,3 +164,13 @@ def forward(cfg, w, tokens, layers_out=None):
             layers_out.append(x.copy())
     h = unit_norm(x, w["final.norm"], eps)
     return linear(h, w["embed"]) * F64(cfg["logit_scale"])
+
+
+def greedy(cfg, w, prompt, n: int):
+    """``n`` tokens after ``prompt``, each the first largest logit of the whole sequence so far."""
+    tokens, out = list(prompt), []
+    for _ in range(n):
+        t = int(np.argmax(forward(cfg, w, tokens)[-1]))
+        out.append(t)
+        tokens.append(t)
+    return out
