@@ -1255,15 +1255,34 @@ class MoEWeight:
 
 
 class MoEPlan:
-    """Which expert every (row, choice) pair takes: ``ids`` int32 [pairs] (None: all take expert 0)."""
+    """Which expert every (row, choice) pair takes: ``ids`` int32 [pairs] (None: all take expert 0),
+    and, once :meth:`group` has run, the pairs laid out expert by expert for the matrix-core product:
+    ``order`` int32 [pairs], ``tiles`` int32 [max_tiles, 4] = (expert, first place in order, pairs, 0),
+    ``n_tiles`` int32 [1] on the device."""
 
     def __init__(self, ids: Optional[torch.Tensor], n_pairs: int, n_experts: int):
         self.ids, self.n_pairs, self.n_experts = ids, n_pairs, n_experts
+        self.tile_rows = int(library.core().sb_moe_tile_rows(n_pairs, n_experts)) if n_pairs else 64
+        self.order = self.tiles = self.n_tiles = None
+        self.max_tiles = 0
+
+    def group(self) -> None:
+        if self.ids is None or self.order is not None or self.n_pairs == 0:
+            return
+        dev = self.ids.device
+        self.max_tiles = self.n_pairs // self.tile_rows + self.n_experts + 1
+        self.order = torch.empty(self.n_pairs, dtype=torch.int32, device=dev)
+        self.tiles = torch.empty((self.max_tiles, 4), dtype=torch.int32, device=dev)
+        self.n_tiles = torch.empty(1, dtype=torch.int32, device=dev)
+        check(library.core().sb_moe_group(_p(self.ids), self.n_pairs, self.n_experts, self.tile_rows, _p(self.order),
+                                          _p(self.tiles), _p(self.n_tiles), _stream()))
 
 
 def moe_plan(ids: Optional[torch.Tensor], n_experts: int, n_pairs: Optional[int] = None, device=None) -> MoEPlan:
     if ids is not None:
+        _dev(ids)
         ids = ids.view(-1)
+        _i32(ids, ids.numel(), "expert numbers")
         n_pairs = ids.numel()
     return MoEPlan(ids, int(n_pairs), int(n_experts))
 
@@ -1271,10 +1290,22 @@ def moe_plan(ids: Optional[torch.Tensor], n_experts: int, n_pairs: Optional[int]
 def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dtype: torch.dtype,
                 limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
     """Y[p] = X[p // x_div] W_e^T for every pair p of ``plan``; a gated weight gives the clamped
-    swish pair of its two halves."""
+    swish pair of its two halves.  bfloat16 operands with an inner size in eights run on the matrix
+    cores, the pairs grouped by expert on the device; everything else takes the plain kernel."""
     if w.experts != plan.n_experts:
         raise KernelLibraryError(f"the plan counts {plan.n_experts} experts, the weight has {w.experts}")
-    return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha)
+    if not (w.fast and x.dtype == torch.bfloat16 and w.w.dtype == torch.bfloat16 and w.n_in % 8 == 0):
+        return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha)
+    _dev(x)
+    if x.dim() != 2 or x.shape[1] != w.n_in or (plan.n_pairs + x_div - 1) // x_div > x.shape[0]:
+        raise KernelLibraryError(f"expert product shapes do not match: x {tuple(x.shape)}, w {tuple(w.w.shape)}, "
+                                 f"{plan.n_pairs} pairs")
+    plan.group()
+    y = torch.empty((plan.n_pairs, w.n_out), dtype=out_dtype, device=x.device)
+    check(library.core().sb_moe_product_bf16(
+        _p(y), _dt(y), _p(x), _p(w.w), _p(plan.order), _p(plan.tiles), _p(plan.n_tiles), plan.max_tiles, plan.tile_rows,
+        plan.n_pairs, int(x_div), w.n_out, w.n_in, 1 if w.gated else 0, float(limit), float(alpha), _stream()))
+    return y
 
 
 def attention_capped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,

@@ -61,6 +61,10 @@ _CORE_SIGNATURES = {
     "sb_attention_capped": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P],
     "sb_moe_max_top": [],
     "sb_moe_route": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "sb_moe_tile_rows": [_I, _I],
+    "sb_moe_group": [_P, _I, _I, _I, _P, _P, _P, _P],
+    "sb_moe_product_bf16_ok": [_I],
+    "sb_moe_product_bf16": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "sb_moe_product": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }
