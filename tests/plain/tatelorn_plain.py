@@ -12,7 +12,7 @@ The design in this file's notation (``n`` tokens, position t = 0 .. n-1, stream 
   x += un(mixer(x), norm1); and, if it has a feed-forward, x += un(ff(x), norm2).
 * mixer ``attention``: q = Wq x, k = Wk x, v = Wv x; every head of q and of k is divided by its root
   mean square (eps inside the root) and multiplied by a weight of the head's size that all heads share
-  (no one-plus here); nothing rotates.  s(t, j) = cap * tanh(scale * q_t.k_j / cap) for j <= t;
+  (no one-plus here); nothing rotates.  s(t, j) = cap * tanh(scale * q_t.k_j / cap) for j <= t (no cap: as it is);
   the weights are exp(s_j) / (1 + sum_j exp(s_j)): a key of score 0 without a value takes part.
   Query head a reads key/value head a // (heads / kv_heads).  Layers that mix values: all of them but
   the first replace v by (1 - lam) v + lam v0, v0 the first such layer's v of the same token, lam the
@@ -63,9 +63,9 @@ def start(cfg, w, tokens, first_position: int = 0):
 
 
 def capped_scores(q, k, scale: float, cap: float):
-    """q [n, dim], k [m, dim] -> [n, m]."""
+    """q [n, dim], k [m, dim] -> [n, m]; a cap of 0 (or none) leaves the scores as they are."""
     s = (q @ k.T) * F64(scale)
-    return F64(cap) * np.tanh(s / F64(cap))
+    return F64(cap) * np.tanh(s / F64(cap)) if cap else s
 
 
 def sink_softmax(s, visible):
