@@ -34,7 +34,11 @@ the same width, head count and feed-forward weight count: prefill of one ``--pro
 and decode of ``--batch`` sequences at that depth, tokens a second, and the time of every kernel of
 one prompt step and one decode step with what it reaches of its roofline (bytes it must move over
 8 TB/s, or flops over the dense bf16 peak, whichever is the larger time).  A table goes to standard
-error, one JSON line to standard output.
+error, one JSON line to standard output.  ``--design tatelorn`` puts the Tatelorn design (blocks that
+norm what their sublayers give back, attention with head norms, capped scores and a sink, routed
+experts) in the Rasizen design's place: eight layers, the first with a dense gated feed-forward, the
+others with eight experts of which a row takes two plus a shared one, so that a row passes as many
+feed-forward weights as in the Qwen2.5 design beside it, and the same heads.
 
 ``--workload forms`` prints a table instead of the line: the decode step (``--batches 1,8``) with
 the qkv, output and down product forced, one at a time, to every form (waves a block x K slices)
@@ -258,6 +262,8 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
     ap.add_argument("--workload", choices=("steady", "mixed", "forms", "designs"), default="steady")
+    ap.add_argument("--design", choices=("rasizen", "tatelorn"), default="rasizen",
+                    help="--workload designs: the design that runs beside the Qwen2.5 design")
     ap.add_argument("--design-sizes", default="2048,4096",
                     help="--workload designs: the widths of the layer sizes to run, comma separated")
     ap.add_argument("--batches", default="1,8", help="--workload forms: the batch sizes, comma separated")
@@ -667,6 +673,23 @@ def qwen_sizes(width, n_layers=8, vocab=32768):
                 vocab_size=vocab, tie_word_embeddings=True)
 
 
+def tatelorn_sizes(width, n_layers=8, vocab=32768, experts=8, top=2):
+    """Layer sizes in the manner of a real model of this width: heads of 128 for keys and for values, a quarter
+    of them kv heads, every layer mixing values; the first layer with a dense feed-forward of 8/3 widths, the
+    others with `experts` experts of one width of which a row takes `top`, and a shared expert that brings a
+    row's feed-forward weights to those of the dense layer."""
+    heads = width // 128
+    inner = (8 * width // 3 + 255) // 256 * 256
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+             "softcap": 30.0, "v_mix": True}
+    routed = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": width, "limit": 7.0},
+              "shared": {"ff": max(256, inner - top * width), "limit": 7.0}}
+    layers = [{"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": inner} if i == 0 else routed}
+              for i in range(n_layers)]
+    return {"architecture": "Tatelorn", "vocab": vocab, "width": width, "max_positions": 1 << 16, "logit_scale": 0.5,
+            "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-6}, "layers": layers}
+
+
 class AllOpsTimer:
     """Times every launching function of ``sonicboom_amd.ops`` between two events, summed by
     (function, what tells its calls apart: a product's matrix, the rows)."""
@@ -674,9 +697,10 @@ class AllOpsTimer:
     SKIP = ("pack_weight", "read_bandwidth", "random_normal", "attention_row_tile", "attention_row_tiles",
             "attention_tall_ok", "attention_mfma_ok", "attention_decode_rope_ok", "gate_code", "reduce_resid_norm_ok",
             "attention_decode_pages_per_wave", "gemm_tile_shape", "gemm_few_rows_kernel", "mingru_chunk_rows",
-            "loaded_paths", "check", "latent_attention_mfma_ok")
+            "loaded_paths", "check", "latent_attention_mfma_ok", "capped_attention_mfma_ok", "moe_max_top", "moe_plan")
     INNER = ("attention_plain", "attention_decode_mfma", "attention_prefill_mfma", "latent_attention_plain",
-             "latent_attention_mfma")      # called by the dispatchers that are timed themselves
+             "latent_attention_mfma", "attention_capped_plain", "attention_capped_mfma",
+             "moe_product_plain")      # called by the dispatchers that are timed themselves
 
     def __init__(self):
         self.records, self._saved = [], {}
@@ -705,6 +729,8 @@ class AllOpsTimer:
                         label = f"{_name} {n}x{k}"
                     elif _name == "head_product":
                         label = f"{_name} {tuple(args[1].shape)}"
+                    elif _name == "moe_product":
+                        label = f"{_name} {args[1].experts}x{args[1].n_out}x{args[1].n_in}{' gated' if args[1].gated else ''}"
                     self.records.append((label, e0, e1))
                 return out
             setattr(ops, name, timed)
@@ -763,6 +789,22 @@ def design_roofline(label, us, calls, rows, depth, batch, width, cfgs):
         nbytes = (batch * depth if decode else rows) * 2 * 2 * cfgs["kvw"] + 4 * rows * H * 128
     elif label == "rope_kv_store":
         nbytes = rows * (H * 128 + 2 * cfgs["kvw"]) * (4 + 2)
+    elif label == "attention_capped":
+        pairs = batch * depth if decode else rows * (rows + 1) // 2
+        flops = 4 * pairs * H * 128
+        nbytes = (batch * depth if decode else rows) * 2 * 2 * cfgs["kvw"] + 4 * rows * H * 128
+    elif label == "headnorm_kv_store":
+        nbytes = rows * (H * 128 + 2 * cfgs["kvw"]) * (4 + 2)
+    elif label == "norm_add":
+        nbytes = rows * width * (4 + 8 + 2)          # one slice of the sublayer's result at least
+    elif label in ("cast", "embed_pos_norm"):
+        nbytes = rows * width * (4 + 2)
+    elif label.startswith("moe_product"):
+        e, n, k = (int(v) for v in label.split()[1].split("x"))
+        m = 2 if "gated" in label else 1
+        pairs = rows * (cfgs["top"] if e > 1 else 1)
+        nbytes = 2 * min(e, pairs) * m * n * k + 2 * pairs * (k + n)
+        flops = 2 * pairs * m * n * k
     if nbytes is None and flops is None:
         return None, ""
     tb, tf = (nbytes or 0) / peak_b, (flops or 0) / peak_f
@@ -778,12 +820,13 @@ def design_comparison(a) -> int:
     rng = np.random.default_rng(0)
     out, table = {}, []
     for width in (int(v) for v in a.design_sizes.split(",")):
-        for design, cfg in (("rasizen", rasizen_sizes(width)), ("qwen2", qwen_sizes(width))):
+        beside = ("rasizen", rasizen_sizes(width)) if a.design == "rasizen" else ("tatelorn", tatelorn_sizes(width))
+        for design, cfg in (beside, ("qwen2", qwen_sizes(width))):
             model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
             heads = width // 128
             cfgs = {"heads": heads, "rank": 512, "rot": 64, "window": 4096 if design == "rasizen" else 1 << 30,
                     "gru": 2 * width, "ff": 4 * width, "kvw": max(1, heads // 4) * 128,
-                    "vocab": cfg.get("vocab", cfg.get("vocab_size"))}
+                    "vocab": cfg.get("vocab", cfg.get("vocab_size")), "top": 2}
             eng = Engine(model, (a.prompt + a.steps + a.warmup + 128) * (a.batch + 1), max_positions=0)
             prompt = [int(t) for t in rng.integers(0, cfg.get("vocab", cfg.get("vocab_size")), size=a.prompt)]
 
@@ -839,7 +882,7 @@ def design_comparison(a) -> int:
     for key, v in out.items():
         print(f"RESULT {key} prefill_tokens_per_s={v['prefill_tokens_per_s']} decode_tokens_per_s={v['decode_tokens_per_s']} "
               f"prefill_ms={v['prefill_ms']} decode_step_ms={v['decode_step_ms']}", file=sys.stderr)
-    print(json.dumps({"workload": "designs", "prompt": a.prompt, "batch": a.batch, "steps": a.steps, "dtype": "bf16",
+    print(json.dumps({"workload": "designs", "design": a.design, "prompt": a.prompt, "batch": a.batch, "steps": a.steps, "dtype": "bf16",
                       "data": "synthetic", "models": out}))
     return 0
 

@@ -124,7 +124,8 @@ class OutNormBlock(Part):
         next block reads it as it is, else None."""
         act = self.rt.act_dtype
         if h is None:
-            h = ops.cast(x, act)
+            left = (getattr(ctx, "shared", None) or {}).pop("stream", None)      # the embedding's own copy of what it made
+            h = left[1] if left is not None and left[0] is x and left[1].dtype == act else ops.cast(x, act)
         last = self.ffn is None
         want = act if not last or isinstance(next_norm, StreamAsItIs) else None
         h = self._join(x, self.mixer.produce(h, ctx, binding), self.mixer_norm, want)

@@ -73,8 +73,11 @@ class PositionalEmbedding(Part):
 
     def forward(self, ids: torch.Tensor, ctx=None) -> torch.Tensor:
         row_pos = ctx.row_pos if self.positions is not None else None
-        x, _ = ops.embed_pos_norm(self.table, ids, self.scale, self.positions, row_pos, self.norm_weight, self.eps,
-                                  self.norm_offset, norm=self.norm_weight is not None)
+        x, copy = ops.embed_pos_norm(self.table, ids, self.scale, self.positions, row_pos, self.norm_weight, self.eps,
+                                     self.norm_offset, norm=self.norm_weight is not None, copy_dtype=self.rt.act_dtype)
+        shared = getattr(ctx, "shared", None)
+        if copy is not None and shared is not None:
+            shared["stream"] = (x, copy)        # the stream in the activation type, for a first block that reads it as it is
         return x
 
 

@@ -168,18 +168,19 @@ def gelu_tanh(g):
 @pytest.mark.parametrize("t", [1, 8, 40, 64, 65, 128, 300])
 def test_gemm_bf16_gate_activations(t):
     """The gate's activation is an argument of every product kernel and of the elementwise
-    kernel: SiLU and the tanh form of GELU, through the stream, the K-splitting and the tiled
-    kernels, against the formula and against torch's own GELU."""
+    kernel: SiLU, the tanh form of GELU and max(g, 0), through the stream, the K-splitting and the
+    tiled kernels, against the formula and against torch's own GELU."""
     from sonicboom_amd import ops
     inner, k = 1040, 264
     x, w = randn(t, k, dtype=BF16), randn(2 * inner, k, dtype=BF16, scale=0.15)
     gu = x.double() @ w.double().T
     g, u = gu[:, :inner], gu[:, inner:]
     assert torch.allclose(gelu_tanh(g), torch.nn.functional.gelu(g, approximate="tanh"), atol=1e-12)
-    want = {"silu": g / (1.0 + torch.exp(-g)) * u, "gelu_tanh": gelu_tanh(g) * u}
+    want = {"silu": g / (1.0 + torch.exp(-g)) * u, "gelu_tanh": gelu_tanh(g) * u, "relu": torch.clamp(g, min=0.0) * u}
     assert (want["silu"] - want["gelu_tanh"]).abs().max() > 0.05          # the two differ visibly
     packed = ops.pack_weight(w.to(DEV), True)
-    for act in ("silu", "gelu_tanh"):
+    assert (want["relu"] - want["gelu_tanh"]).abs().max() > 0.05
+    for act in ("silu", "gelu_tanh", "relu"):
         for which in ("stream", "skinny", "tiled"):
             if (which == "stream" and t > 128) or (which == "skinny" and t > 64):
                 continue
@@ -189,7 +190,7 @@ def test_gemm_bf16_gate_activations(t):
         got = ops.gate_mul(gu.float().to(DEV), F32, act)
         close(got, want[act], atol=1e-5, rtol=1e-5, what=f"{act}, elementwise")
     with pytest.raises(ops.KernelLibraryError, match="unknown gate activation"):
-        ops.gate_mul(gu.float().to(DEV), F32, "relu")
+        ops.gate_mul(gu.float().to(DEV), F32, "softsign")
 
 
 @pytest.mark.parametrize("shape", [0, 1, 2])
