@@ -14,9 +14,10 @@
 //         row r of an S^T tile stands for key 8 (r / 4) + 4 t + r % 4 of a half page (t the tile), so
 //         the eight probabilities a lane holds after two tiles are eight consecutive keys.
 //
-// Softmax in float32, running maximum and sum per query column; a sink starts the maximum at 0 and
-// the sum at 1.  Steps of few rows share the pages of a sequence out over `chunks` blocks, which
-// leave (unnormed result, maximum, sum) for sb_cattn_merge.
+// Softmax in float32, running maximum and sum per query column, scores kept times log2(e) so that the
+// weights are powers of two; a sink starts the maximum at 0 and the sum at 1.  Steps of few rows
+// share the pages of a sequence out over `chunks` blocks, which leave (unnormed result, maximum,
+// sum) for the merge kernel.
 #include "mfma.h"
 
 #if !defined(SB_KEY_DIM) || !defined(SB_VALUE_DIM)
@@ -58,12 +59,16 @@ struct Args {
   const int32_t *row_pos, *tiles;
   int n_rows, heads_q, heads_kv;
   float scale, softcap; int window, sink, chunk_pages;
+  unsigned round_blocks;       // blocks the GPU takes one of per CU
 };
 
-// softcap * tanh(s / softcap) with the fast exponential: tanh(x) = 1 - 2 / (exp(2x) + 1)
-__device__ __forceinline__ float capped(float s, float cap, float inv_cap) {
-  const float x = fminf(fmaxf(s * inv_cap, -15.0f), 15.0f);
-  return cap * (1.0f - 2.0f / (__expf(2.0f * x) + 1.0f));
+constexpr float kLog2e = 1.4426950408889634f;
+
+// softcap * tanh(s / softcap) by the hardware's exponential and reciprocal: tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1).
+// two_log2e_over_cap = 2 log2(e) / softcap.
+__device__ __forceinline__ float capped(float s, float cap, float two_log2e_over_cap) {
+  const float t = fminf(s * two_log2e_over_cap, 60.0f);          // 2^60 + 1 is 2^60 in float32: tanh is 1 by then
+  return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(t) + 1.0f));
 }
 
 __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
@@ -75,7 +80,13 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   const int hg = hz * NW + wave;                  // the wave's head within the group
   const bool has_head = hg < group;
   const int h = kvh * group + (has_head ? hg : 0);
-  const int32_t *tile = a.tiles + size_t(blockIdx.x) * 4;
+  // Later rows of a sequence see more pages.  All blocks of a prompt step are usually resident at once, a CU
+  // holding blocks a whole round of the GPU apart: every other round of 256 blocks walks the tiles from
+  // the far end, so that a CU's blocks are a heavy and a light one.
+  // (one direction for all blocks of a (head group, chunk): every tile is taken once)
+  const unsigned first_of_row = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int tile_no = ((first_of_row / a.round_blocks) & 1) ? int(gridDim.x) - 1 - int(blockIdx.x) : int(blockIdx.x);
+  const int32_t *tile = a.tiles + size_t(tile_no) * 4;
   const int r0 = tile[0], nr = tile[1], seq = tile[2];
   const int chunk = blockIdx.z;
   const int p0 = a.row_pos[r0], p_last = p0 + nr - 1;
@@ -104,7 +115,9 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   floatx4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-  const float inv_cap = a.softcap > 0.0f ? 1.0f / a.softcap : 0.0f;
+  const float cap_arg = a.softcap > 0.0f ? 2.0f * kLog2e / a.softcap : 0.0f;
+  // scores are kept times log2(e), so that the weights are powers of two: the sink's score stays 0
+  const float scale2 = a.scale * kLog2e, cap2 = a.softcap * kLog2e;
 
   uint4 kreg[kKeyLoads], vreg[kValLoads];
   auto fetch = [&](int c) {
@@ -149,6 +162,8 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
     for (int hp = 0; hp < 2; ++hp) {
       const int first = c * SB_PAGE + 32 * hp;          // position of the half page's first key
       if (first > p_last || first + 31 < lo) continue;  // uniform over the block
+      // every row of the tile sees every key of this half page: no score needs a test (uniform)
+      const bool whole = nr == kTile && first + 31 <= p0 && (a.window == 0 || first >= p_last - a.window + 1);
       floatx4_t s[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
@@ -170,20 +185,21 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int j = first + 8 * g + 4 * t + i;
-          float v = s[t][i] * a.scale;
-          if (a.softcap > 0.0f) v = capped(v, a.softcap, inv_cap);
-          const bool visible = col < nr && j <= q_pos && j >= q_lo;
+          float v;
+          if (a.softcap > 0.0f) v = capped(s[t][i] * a.scale, cap2, cap_arg);
+          else v = s[t][i] * scale2;
+          const bool visible = whole || (col < nr && j <= q_pos && j >= q_lo);
           v = visible ? v : neg_inf;
           sc[4 * t + i] = v;
           mx = fmaxf(mx, v);
         }
       mx = max_over_lane_groups(mx);
       const float m_new = fmaxf(m, mx);
-      const float alpha = m == neg_inf ? 0.0f : __expf(m - m_new);
+      const float alpha = m == neg_inf ? 0.0f : __builtin_amdgcn_exp2f(m - m_new);
       float psum = 0.0f, p[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = sc[e] == neg_inf ? 0.0f : __expf(sc[e] - m_new);
+        p[e] = sc[e] == neg_inf ? 0.0f : __builtin_amdgcn_exp2f(sc[e] - m_new);
         psum += p[e];
       }
       l = l * alpha + psum;
@@ -244,7 +260,7 @@ merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const f
   for (int c = 0; c < chunks; ++c) {
     const float mc = part_ml[(size_t(c) * n_heads + rh) * 2];
     if (mc == -__builtin_inff()) continue;
-    const float w = __expf(mc - big);
+    const float w = __builtin_amdgcn_exp2f(mc - big);          // the maxima are kept times log2(e)
     num = fmaf(w, part_o[size_t(c) * n_heads * DV + idx], num);
     den = fmaf(w, part_ml[(size_t(c) * n_heads + rh) * 2 + 1], den);
   }
@@ -284,6 +300,7 @@ extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, cons
   a.page_table = page_table; a.max_pages = max_pages; a.n_pages = n_pages; a.row_pos = row_pos; a.tiles = tiles;
   a.n_rows = n_rows; a.heads_q = heads_q; a.heads_kv = heads_kv; a.scale = scale; a.softcap = softcap;
   a.window = window; a.sink = sink; a.chunk_pages = chunks == 1 ? 0 : chunk_pages;
+  a.round_blocks = unsigned(sb::cu_count());
   capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups, chunks), kThreads, 0, s>>>(a);
   int st = sb::check_launch("sb_cattn_bf16");
   if (st != SB_OK || chunks == 1) return st;

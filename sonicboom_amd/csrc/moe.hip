@@ -5,6 +5,8 @@
 //                   softmax over the chosen scores alone; with has_gate also sigmoid(z[n_experts]),
 //                   the multiplier of an expert that every row takes.
 //                   ids int32 [rows, top]; weights f32 [rows, top + 1] (the last: the gate, or 0).
+//   sb_moe_router   the router's product (float32 sums of a float32 matrix against rows of either type)
+//                   and sb_moe_route's choice in one launch, a block a row.
 //   sb_moe_product  Y[p,:] = X[p / x_div,:] W_e^T for every pair p = (row, choice), e = ids[p]
 //                   (ids NULL: expert 0 for all); gated: W_e = [W_gate; W_up] and
 //                   Y = g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = u cut to +-limit.
@@ -16,12 +18,10 @@ namespace {
 
 constexpr int kMaxTop = 16;
 
-__global__ void __launch_bounds__(64)
-moe_route_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const float *__restrict__ z, int n_rows,
-                 int stride, int n_experts, int top, int has_gate) {
-  const int r = blockIdx.x * 64 + threadIdx.x;
-  if (r >= n_rows) return;
-  const float *zr = z + size_t(r) * stride;
+// One row's choice from its scores zr: the `top` largest in falling order (ties to the lower
+// number), the softmax over them, the gate.
+__device__ __forceinline__ void route_row(int32_t *__restrict__ ids, float *__restrict__ weights, const float *zr, int r,
+                                          int n_experts, int top, int has_gate) {
   int chosen[kMaxTop];
   float score[kMaxTop];
   for (int k = 0; k < top; ++k) {
@@ -45,6 +45,87 @@ moe_route_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const f
     weights[size_t(r) * (top + 1) + k] = w[k] / sum;
   }
   weights[size_t(r) * (top + 1) + top] = has_gate ? 1.0f / (1.0f + expf(-zr[n_experts])) : 0.0f;
+}
+
+__global__ void __launch_bounds__(64)
+moe_route_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const float *__restrict__ z, int n_rows,
+                 int stride, int n_experts, int top, int has_gate) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
+  if (r >= n_rows) return;
+  route_row(ids, weights, z + size_t(r) * stride, r, n_experts, top, has_gate);
+}
+
+// The router's product and the choice in one launch: a block a row.  z_e = sum_k h[k] w[e][k] in
+// float32, eight experts at a time; a thread takes the k of its place in every stretch of 256 (in
+// eights when the row allows, so that a pass's loads are all in flight together), in ascending
+// order, then a fixed butterfly over the wave and the four waves in ascending order: a row's scores
+// depend on the row alone.  w is float32 [n_experts (+ 1), n_in], the last row the gate of the expert
+// that every row takes.
+__device__ __forceinline__ void load8(const float *p, float (&v)[8]) {
+  const float4 a = reinterpret_cast<const float4 *>(p)[0], b = reinterpret_cast<const float4 *>(p)[1];
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t *p, float (&v)[8]) {
+  const uint4 a = *reinterpret_cast<const uint4 *>(p);
+  const uint32_t u[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(u[i] << 16); v[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u); }
+}
+
+template <typename TX>
+__global__ void __launch_bounds__(256)
+moe_router_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const TX *__restrict__ h,
+                  const float *__restrict__ w, int n_rows, int n_in, int n_experts, int top, int has_gate) {
+  extern __shared__ float zs[];                 // [n_z] scores, then [4][8] the waves' sums of a pass
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int r = blockIdx.x;
+  const int n_z = n_experts + (has_gate ? 1 : 0);
+  float *z = zs, *part = zs + n_z;
+  const TX *hr = h + size_t(r) * n_in;
+  const bool vec = n_in % 8 == 0 && (reinterpret_cast<uintptr_t>(hr) % 16 == 0) && (reinterpret_cast<uintptr_t>(w) % 16 == 0);
+  for (int e0 = 0; e0 < n_z; e0 += 8) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      for (int k = tid * 8; k < n_in; k += 256 * 8) {
+        float x[8];
+        load8(hr + k, x);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (e0 + j < n_z) {
+            float wv[8];
+            load8(w + size_t(e0 + j) * n_in + k, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[j] = fmaf(x[i], wv[i], acc[j]);
+          }
+        }
+      }
+    } else {
+      for (int k = tid; k < n_in; k += 256) {
+        const float x = ld_f(hr, k);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (e0 + j < n_z) acc[j] = fmaf(x, w[size_t(e0 + j) * n_in + k], acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float t = wave_sum(acc[j]);
+      if (lane == 0) part[wave * 8 + j] = t;
+    }
+    __syncthreads();
+    if (tid < 8 && e0 + tid < n_z) z[e0 + tid] = ((part[tid] + part[8 + tid]) + part[16 + tid]) + part[24 + tid];
+    __syncthreads();
+  }
+  if (tid == 0) route_row(ids, weights, z, r, n_experts, top, has_gate);
+}
+
+template <typename TO>
+__global__ void swish_clamp_kernel(TO *__restrict__ out, const float *__restrict__ gu, int width, size_t n, float limit,
+                                   float alpha) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const size_t t = idx / width, i = idx % width;
+  st_f(out, idx, swish_clamp_mul(gu[t * 2 * width + i], gu[t * 2 * width + width + i], limit, alpha));
 }
 
 template <typename TX, typename TW, typename TY>
@@ -87,6 +168,35 @@ extern "C" int sb_moe_route(int32_t *ids, float *weights, const float *z, int n_
   if (n_rows == 0) return SB_OK;
   moe_route_kernel<<<(n_rows + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, z, n_rows, stride, n_experts, top, has_gate);
   return sb::check_launch("sb_moe_route");
+}
+
+extern "C" int sb_moe_router(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                             int n_in, int n_experts, int top, int has_gate, void *stream) {
+  SB_REQUIRE(ids && weights && h && w, "sb_moe_router: null pointer");
+  SB_REQUIRE(n_rows >= 0 && n_in > 0 && n_experts > 0 && top > 0 && top <= n_experts && sb::valid_dtype(h_dtype),
+             "sb_moe_router: bad sizes rows=%d in=%d experts=%d top=%d", n_rows, n_in, n_experts, top);
+  SB_SUPPORT(top <= kMaxTop && n_experts < 2048, "sb_moe_router: %d choices of %d experts are more than %d of 2047", top,
+             n_experts, kMaxTop);
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = size_t(n_experts + 1 + 32) * sizeof(float);
+  const unsigned blocks = n_rows;
+  if (h_dtype == SB_F32) moe_router_kernel<float><<<blocks, 256, lds, s>>>(ids, weights, (const float *)h, w, n_rows, n_in, n_experts, top, has_gate);
+  else moe_router_kernel<bf16_t><<<blocks, 256, lds, s>>>(ids, weights, (const bf16_t *)h, w, n_rows, n_in, n_experts, top, has_gate);
+  return sb::check_launch("sb_moe_router");
+}
+
+// out[t,i] = g' sigmoid(alpha g') (u' + 1), g' = min(gu[t,i], limit), u' = gu[t,width+i] cut to +-limit; gu f32 [t, 2*width]
+extern "C" int sb_swish_clamp_mul(void *out, int out_dtype, const float *gu, int n_rows, int width, float limit, float alpha,
+                                  void *stream) {
+  SB_REQUIRE(out && gu, "sb_swish_clamp_mul: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && sb::valid_dtype(out_dtype), "sb_swish_clamp_mul: bad sizes rows=%d width=%d", n_rows, width);
+  const size_t n = size_t(n_rows) * width;
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == SB_F32) swish_clamp_kernel<float><<<unsigned((n + 255) / 256), 256, 0, s>>>((float *)out, gu, width, n, limit, alpha);
+  else swish_clamp_kernel<bf16_t><<<unsigned((n + 255) / 256), 256, 0, s>>>((bf16_t *)out, gu, width, n, limit, alpha);
+  return sb::check_launch("sb_swish_clamp_mul");
 }
 
 extern "C" int sb_moe_product(void *y, int y_dtype, const void *x, int x_dtype, const void *w, int w_dtype,

@@ -112,17 +112,21 @@ __global__ void __launch_bounds__(kThreads) moe_product_kernel(Args a) {
       b_src[i] = n < a.n_out ? we + size_t(n) * a.n_in : nullptr;
     }
   }
-  uint4 areg[kALoads], breg[kBLoads];
-  auto fetch = [&](int k0) {
+  // the low tile (few pairs an expert: decode steps, whose few blocks a CU would wait for memory once
+  // per k tile) keeps two k tiles' loads in flight while a third is multiplied; the high tile, whose
+  // accumulators take the registers, one
+  constexpr int DEPTH = MT <= 2 ? 2 : 1;
+  uint4 areg[DEPTH][kALoads], breg[DEPTH][kBLoads];
+  auto fetch = [&](uint4 *ar, uint4 *br, int k0) {
 #pragma unroll
     for (int i = 0; i < kALoads; ++i) {
       const int k = k0 + 8 * a_chunk[i];
-      areg[i] = (a_src[i] && k < a.n_in) ? *reinterpret_cast<const uint4 *>(a_src[i] + k) : make_uint4(0u, 0u, 0u, 0u);
+      ar[i] = (a_src[i] && k < a.n_in) ? *reinterpret_cast<const uint4 *>(a_src[i] + k) : make_uint4(0u, 0u, 0u, 0u);
     }
 #pragma unroll
     for (int i = 0; i < kBLoads; ++i) {
       const int k = k0 + 8 * b_chunk[i];
-      breg[i] = (b_src[i] && k < a.n_in) ? *reinterpret_cast<const uint4 *>(b_src[i] + k) : make_uint4(0u, 0u, 0u, 0u);
+      br[i] = (b_src[i] && k < a.n_in) ? *reinterpret_cast<const uint4 *>(b_src[i] + k) : make_uint4(0u, 0u, 0u, 0u);
     }
   };
 
@@ -132,15 +136,14 @@ __global__ void __launch_bounds__(kThreads) moe_product_kernel(Args a) {
 #pragma unroll
     for (int f = 0; f < 4; ++f) acc[i][f] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  fetch(0);
-  for (int k0 = 0; k0 < a.n_in; k0 += BK) {
+  auto step = [&](uint4 *ar, uint4 *br, int k0) {
     __syncthreads();        // the tile before has been read
 #pragma unroll
-    for (int i = 0; i < kALoads; ++i) { const int idx = tid + i * kThreads; a_lds[lds_at(idx >> 3, idx & 7)] = areg[i]; }
+    for (int i = 0; i < kALoads; ++i) { const int idx = tid + i * kThreads; a_lds[lds_at(idx >> 3, idx & 7)] = ar[i]; }
 #pragma unroll
-    for (int i = 0; i < kBLoads; ++i) { const int idx = tid + i * kThreads; b_lds[lds_at(idx >> 3, idx & 7)] = breg[i]; }
+    for (int i = 0; i < kBLoads; ++i) { const int idx = tid + i * kThreads; b_lds[lds_at(idx >> 3, idx & 7)] = br[i]; }
     __syncthreads();
-    if (k0 + BK < a.n_in) fetch(k0 + BK);
+    if (k0 + DEPTH * BK < a.n_in) fetch(ar, br, k0 + DEPTH * BK);
 #pragma unroll
     for (int ks = 0; ks < BK / 32; ++ks) {
       const int c = 4 * ks + g;
@@ -154,6 +157,12 @@ __global__ void __launch_bounds__(kThreads) moe_product_kernel(Args a) {
 #pragma unroll
         for (int f = 0; f < 4; ++f) acc[i][f] = mfma16(af[i], bf[f], acc[i][f]);
     }
+  };
+  fetch(areg[0], breg[0], 0);
+  if (DEPTH == 2 && BK < a.n_in) fetch(areg[DEPTH - 1], breg[DEPTH - 1], BK);
+  for (int k0 = 0; k0 < a.n_in; k0 += DEPTH * BK) {
+    step(areg[0], breg[0], k0);
+    if (DEPTH == 2 && k0 + BK < a.n_in) step(areg[DEPTH - 1], breg[DEPTH - 1], k0 + BK);
   }
 
   // acc[i][f][e]: pair row 16 MT wr + 16 i + 4 g + e, matrix row (of the wave's 64) 16 f + col

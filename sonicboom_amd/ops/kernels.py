@@ -1388,6 +1388,32 @@ def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool):
     return ids, weights
 
 
+def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_gate: bool):
+    """The router in one launch: z = h w^T in float32 (``w`` float32 [n_experts (+ 1 with
+    ``has_gate``), width], ``h`` rows of either type), then what :func:`moe_route` gives."""
+    _dev(h, w)
+    if w.dtype != torch.float32 or w.dim() != 2 or h.dim() != 2 or h.shape[1] != w.shape[1] \
+            or w.shape[0] != n_experts + (1 if has_gate else 0):
+        raise KernelLibraryError(f"the router's matrix must be float32 [{n_experts + (1 if has_gate else 0)}, {h.shape[-1]}]")
+    n = h.shape[0]
+    ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((n, top + 1), dtype=torch.float32, device=h.device)
+    check(library.core().sb_moe_router(_p(ids), _p(weights), _p(h), _dt(h), _p(w), n, h.shape[1], int(n_experts), int(top),
+                                       1 if has_gate else 0, _stream()))
+    return ids, weights
+
+
+def swish_clamp_mul(gu: torch.Tensor, out_dtype: torch.dtype, limit: float, alpha: float) -> torch.Tensor:
+    """g' sigmoid(alpha g') (u' + 1) for gu = [g | u] float32 [n, 2w], g' = min(g, limit), u' = u cut to +-limit."""
+    _dev(gu)
+    if gu.dtype != torch.float32 or gu.dim() != 2 or gu.shape[1] % 2:
+        raise KernelLibraryError("the pair's input must be float32 [rows, 2*width]")
+    n, w2 = gu.shape
+    out = torch.empty((n, w2 // 2), dtype=out_dtype, device=gu.device)
+    check(library.core().sb_swish_clamp_mul(_p(out), _dt(out), _p(gu), n, w2 // 2, float(limit), float(alpha), _stream()))
+    return out
+
+
 def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tensor], n_pairs: int, x_div: int,
                       out_dtype: torch.dtype, gated: bool = False, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
     """Y[p] = X[p // x_div] W_e^T, e = ids[p] (None: expert 0), by the plain kernel.  ``w``

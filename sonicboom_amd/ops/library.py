@@ -65,6 +65,8 @@ _CORE_SIGNATURES = {
     "sb_moe_group": [_P, _I, _I, _I, _P, _P, _P, _P],
     "sb_moe_product_bf16_ok": [_I],
     "sb_moe_product_bf16": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+    "sb_moe_router": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "sb_swish_clamp_mul": [_P, _I, _P, _I, _I, _F, _F, _P],
     "sb_moe_product": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }

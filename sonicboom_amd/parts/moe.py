@@ -8,7 +8,7 @@
     u' = W_up f cut to [-limit, limit]                                  ("swish_clamp")
 
 The router runs in float32 whatever the model's type (its matrix, with the shared expert's gate
-row under it, is kept in float32 and takes the plain product).  Choice and weights are made on the
+row under it, is kept in float32; one kernel makes the scores and the choice).  Choice and weights are made on the
 device, and the experts' products find their rows there too: nothing of a step depends on a value the
 host has seen, so a decode step can be recorded and replayed.  The experts' matrices are stacked
 when the part is built: [experts, 2 * inner, width] (gate over up) and [experts, width, inner].
@@ -78,31 +78,33 @@ class MoEFFN(Part):
         rows = [tensors["router"].float()]
         if self.shared_inner:
             rows.append(tensors["shared.sg"].float().reshape(1, self.width))
-        self.router = Linear(torch.cat(rows, dim=0), None, rt.fast_kernels)          # float32: the plain product
+        self.router = torch.cat(rows, dim=0).contiguous()        # float32, the shared expert's gate row last
         self.w_in = ops.MoEWeight(_stack([torch.cat([tensors[f"e{e}.gate"], tensors[f"e{e}.up"]], dim=0)
                                           for e in range(self.experts)]), gated=True, fast=rt.fast_kernels)
         self.w_out = ops.MoEWeight(_stack([tensors[f"e{e}.down"] for e in range(self.experts)]), fast=rt.fast_kernels)
+        # the expert that every row takes is a dense feed-forward: the framework's own products, with the
+        # clamped pair applied to the float32 result of the stacked one
         self.s_in = self.s_out = None
         if self.shared_inner:
-            self.s_in = ops.MoEWeight(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0).unsqueeze(0).contiguous(),
-                                      gated=True, fast=rt.fast_kernels)
-            self.s_out = ops.MoEWeight(tensors["shared.down"].unsqueeze(0).contiguous(), fast=rt.fast_kernels)
+            g, u = tensors["shared.gate"], tensors["shared.up"]
+            if g.dtype != u.dtype:
+                g, u = g.float(), u.float()
+            self.s_in = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels)
+            self.s_out = Linear(tensors["shared.down"], None, rt.fast_kernels)
 
     def produce(self, h, ctx):
         """The pairs' results [rows, top, width] with their weights, and the shared expert's with its
         gate, for the pass that adds them up."""
         act = self.rt.act_dtype
         n = h.shape[0]
-        z = self.router(h, torch.float32)                                  # [n, experts (+ 1)]
-        ids, weights = ops.moe_route(z, self.experts, self.top, has_gate=bool(self.shared_inner))
+        ids, weights = ops.moe_router(h, self.router, self.experts, self.top, has_gate=bool(self.shared_inner))
         plan = ops.moe_plan(ids, self.experts)
         mid = ops.moe_product(h, self.w_in, plan, self.top, act, self.limit, self.alpha)       # [n * top, inner]
         out = ops.moe_product(mid, self.w_out, plan, 1, torch.float32)                         # [n * top, width]
         branch = Branch(out.view(n, self.top, self.width), by_row=True, part_weights=weights[:, : self.top])
         if self.shared_inner:
-            every = ops.moe_plan(None, 1, n_pairs=n, device=h.device)
-            smid = ops.moe_product(h, self.s_in, every, 1, act, self.shared_limit, self.alpha)
-            branch.extra = ops.moe_product(smid, self.s_out, every, 1, torch.float32)
+            smid = ops.swish_clamp_mul(self.s_in(h, torch.float32), act, self.shared_limit, self.alpha)
+            branch.extra = self.s_out(smid, torch.float32)
             branch.extra_weights = weights[:, self.top:]
         return branch
 
