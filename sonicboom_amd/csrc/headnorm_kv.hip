@@ -24,8 +24,28 @@ struct Args {
   int heads_q, heads_kv, dk, dv, store;
 };
 
-template <typename TQ, typename TC>
-__global__ void __launch_bounds__(256) headnorm_kv_store_kernel(Args a) {
+constexpr int kMaxSlices = 8;      // slices whose loads the unrolled loops ask for together (more: the plain loop)
+
+// the sum over the slices of one number of a row: all loads asked for before any is added
+__device__ __forceinline__ float sum_slices(const float *p, int n_slices, size_t slice_stride) {
+  if (n_slices == 1) return p[0];
+  if (n_slices <= kMaxSlices) {
+    float in[kMaxSlices];
+#pragma unroll
+    for (int s = 0; s < kMaxSlices; ++s) in[s] = p[size_t(min(s, n_slices - 1)) * slice_stride];
+    float v = 0.0f;
+#pragma unroll
+    for (int s = 0; s < kMaxSlices; ++s)
+      if (s < n_slices) v += in[s];
+    return v;
+  }
+  float v = 0.0f;
+  for (int s = 0; s < n_slices; ++s) v += p[s * slice_stride];
+  return v;
+}
+
+template <typename TQ, typename TC, int THREADS>
+__global__ void __launch_bounds__(THREADS) headnorm_kv_store_kernel(Args a) {
   const int row = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float *src = a.qkv + size_t(row) * a.row_stride;
   int page = -1, slot = 0;
@@ -36,7 +56,7 @@ __global__ void __launch_bounds__(256) headnorm_kv_store_kernel(Args a) {
     if (page >= a.n_pages) page = -1;
   }
   const int units = a.heads_q + (a.store ? a.heads_kv : 0);
-  for (int u = wave; u < units; u += 4) {
+  for (int u = wave; u < units; u += THREADS / 64) {
     const int col = u * a.dk;
     float v[kMaxHead / 64];
     double sq = 0.0;
@@ -45,7 +65,7 @@ __global__ void __launch_bounds__(256) headnorm_kv_store_kernel(Args a) {
       const int d = lane + 64 * i;
       v[i] = 0.0f;
       if (d < a.dk) {
-        for (int s = 0; s < a.n_slices; ++s) v[i] += src[s * a.slice_stride + col + d];
+        v[i] = sum_slices(src + col + d, a.n_slices, a.slice_stride);
         sq += double(v[i] * v[i]);
       }
     }
@@ -66,9 +86,8 @@ __global__ void __launch_bounds__(256) headnorm_kv_store_kernel(Args a) {
   if (!a.store) return;
   const int v0 = (a.heads_q + a.heads_kv) * a.dk, nv = a.heads_kv * a.dv;
   const float lam = a.v_first ? ld_dyn(a.lam, a.lam_dtype, 0) : 0.0f;
-  for (int e = threadIdx.x; e < nv; e += 256) {
-    float v = 0.0f;
-    for (int s = 0; s < a.n_slices; ++s) v += src[s * a.slice_stride + v0 + e];
+  for (int e = threadIdx.x; e < nv; e += THREADS) {
+    float v = sum_slices(src + v0 + e, a.n_slices, a.slice_stride);
     if (a.v_out) a.v_out[size_t(row) * nv + e] = v;
     if (a.v_first) v = (1.0f - lam) * v + lam * a.v_first[size_t(row) * nv + e];
     if (page >= 0)
@@ -99,9 +118,11 @@ extern "C" int sb_headnorm_kv_store(void *q_out, int q_dtype, const float *qkv, 
                row_pos, row_seq, page_table, max_pages, n_pages, k_cache, v_cache, heads_q, heads_kv, dk, dv, store ? 1 : 0};
   hipStream_t s = (hipStream_t)stream;
   const bool qf = q_dtype == SB_F32, cf = !store || cache_dtype == SB_F32;
-  if (qf && cf) headnorm_kv_store_kernel<float, float><<<n_rows, 256, 0, s>>>(a);
-  else if (qf) headnorm_kv_store_kernel<float, bf16_t><<<n_rows, 256, 0, s>>>(a);
-  else if (cf && store) headnorm_kv_store_kernel<bf16_t, float><<<n_rows, 256, 0, s>>>(a);
-  else headnorm_kv_store_kernel<bf16_t, bf16_t><<<n_rows, 256, 0, s>>>(a);
+  // (a wave a head: the sums do not depend on the block's size, so few rows may take more waves a row)
+  if (qf && cf) headnorm_kv_store_kernel<float, float, 256><<<n_rows, 256, 0, s>>>(a);
+  else if (qf) headnorm_kv_store_kernel<float, bf16_t, 256><<<n_rows, 256, 0, s>>>(a);
+  else if (cf && store) headnorm_kv_store_kernel<bf16_t, float, 256><<<n_rows, 256, 0, s>>>(a);
+  else if (n_rows <= 64) headnorm_kv_store_kernel<bf16_t, bf16_t, 1024><<<n_rows, 1024, 0, s>>>(a);
+  else headnorm_kv_store_kernel<bf16_t, bf16_t, 256><<<n_rows, 256, 0, s>>>(a);
   return sb::check_launch("sb_headnorm_kv_store");
 }

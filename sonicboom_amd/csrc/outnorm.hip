@@ -78,6 +78,115 @@ __global__ void __launch_bounds__(kThreads) norm_add_kernel(AddArgs a) {
   }
 }
 
+// The same pass for rows in fours that fit a block's registers: a thread keeps KEEP groups of four, asks
+// for every slice of all of them before it adds any (slices past the last read the last again with a
+// multiplier of zero: no branch stands between the loads), and the row never goes through LDS.  Few rows:
+// 1024 threads a row, so that a row's loads are one round trip; many rows: 256.
+constexpr int kMaxFastSlices = 8;
+
+template <int THREADS>
+__device__ __forceinline__ double block_sum_n(double part) {
+  __shared__ double wave_part[THREADS / 64];
+  part = wave_sum(part);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int k = 0; k < THREADS / 64; ++k) total += wave_part[k];
+  return total;
+}
+
+template <typename TC, int THREADS, int KEEP, int SL>      // SL: slices the unrolled loops ask for (>= the row's)
+__global__ void __launch_bounds__(THREADS) norm_add_fast_kernel(AddArgs a) {
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int n_groups = a.width / 4;
+  const float4 *p = reinterpret_cast<const float4 *>(a.part + size_t(t) * a.row_stride);
+  const size_t slice4 = a.slice_stride / 4;
+  float sw[SL];
+#pragma unroll
+  for (int s = 0; s < SL; ++s)
+    sw[s] = s < a.n_slices ? (a.part_w ? a.part_w[size_t(t) * a.part_w_stride + s] : 1.0f) : 0.0f;
+  const float ew = a.extra ? (a.extra_w ? a.extra_w[size_t(t) * a.extra_w_stride] : 1.0f) : 0.0f;
+  float4 v[KEEP], xv[KEEP], ev[KEEP], in[KEEP][SL];
+  const float4 *x4 = reinterpret_cast<const float4 *>(a.x + size_t(t) * a.width);
+  const float4 *e4 = a.extra ? reinterpret_cast<const float4 *>(a.extra + size_t(t) * a.width) : x4;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int g = min(tid + i * THREADS, n_groups - 1);
+#pragma unroll
+    for (int s = 0; s < SL; ++s) in[i][s] = p[size_t(min(s, a.n_slices - 1)) * slice4 + g];
+    xv[i] = x4[g];
+    ev[i] = e4[g];
+  }
+  double sq = 0.0;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (a.part_w) {
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        acc.x = fmaf(sw[s], in[i][s].x, acc.x); acc.y = fmaf(sw[s], in[i][s].y, acc.y);
+        acc.z = fmaf(sw[s], in[i][s].z, acc.z); acc.w = fmaf(sw[s], in[i][s].w, acc.w);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < SL; ++s)
+        if (s < a.n_slices) { acc.x += in[i][s].x; acc.y += in[i][s].y; acc.z += in[i][s].z; acc.w += in[i][s].w; }
+    }
+    if (a.extra) {
+      acc.x = fmaf(ew, ev[i].x, acc.x); acc.y = fmaf(ew, ev[i].y, acc.y);
+      acc.z = fmaf(ew, ev[i].z, acc.z); acc.w = fmaf(ew, ev[i].w, acc.w);
+    }
+    v[i] = acc;
+    if (tid + i * THREADS < n_groups)
+      sq += double(acc.x * acc.x) + double(acc.y * acc.y) + double(acc.z * acc.z) + double(acc.w * acc.w);
+  }
+  const float inv = a.do_norm ? inv_rms(block_sum_n<THREADS>(sq), a.width, a.eps) : 1.0f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int g = tid + i * THREADS;
+    if (g >= n_groups) continue;
+    float m[4] = {1.f, 1.f, 1.f, 1.f};
+    if (a.do_norm && a.w) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) m[e] = a.offset + ld_dyn(a.w, a.w_dtype, 4 * g + e);
+    }
+    float4 o;
+    o.x = xv[i].x + (v[i].x * inv) * m[0]; o.y = xv[i].y + (v[i].y * inv) * m[1];
+    o.z = xv[i].z + (v[i].z * inv) * m[2]; o.w = xv[i].w + (v[i].w * inv) * m[3];
+    reinterpret_cast<float4 *>(a.x + size_t(t) * a.width)[g] = o;
+    if (a.copy) {
+      TC *cr = (TC *)a.copy + size_t(t) * a.width + 4 * g;
+      if constexpr (sizeof(TC) == 2) {
+        uint2 w2;
+        w2.x = uint32_t(f32_to_bf16(o.x)) | uint32_t(f32_to_bf16(o.y)) << 16;
+        w2.y = uint32_t(f32_to_bf16(o.z)) | uint32_t(f32_to_bf16(o.w)) << 16;
+        *reinterpret_cast<uint2 *>(cr) = w2;
+      } else {
+        *reinterpret_cast<float4 *>(cr) = o;
+      }
+    }
+  }
+}
+
+template <typename TC, int THREADS, int SL>
+bool launch_fast_sl(const AddArgs &a, int n_rows, hipStream_t s) {
+  const int need = (a.width / 4 + THREADS - 1) / THREADS;
+  if (need <= 1) norm_add_fast_kernel<TC, THREADS, 1, SL><<<n_rows, THREADS, 0, s>>>(a);
+  else if (need <= 2) norm_add_fast_kernel<TC, THREADS, 2, SL><<<n_rows, THREADS, 0, s>>>(a);
+  else if (need <= 4 && THREADS == 256 && SL <= 4) norm_add_fast_kernel<TC, THREADS, 4, SL><<<n_rows, THREADS, 0, s>>>(a);
+  else return false;
+  return true;
+}
+
+template <typename TC, int THREADS>
+bool launch_fast(const AddArgs &a, int n_rows, hipStream_t s) {
+  if (a.n_slices <= 1) return launch_fast_sl<TC, THREADS, 1>(a, n_rows, s);
+  if (a.n_slices <= 2) return launch_fast_sl<TC, THREADS, 2>(a, n_rows, s);
+  if (a.n_slices <= 4) return launch_fast_sl<TC, THREADS, 4>(a, n_rows, s);
+  return launch_fast_sl<TC, THREADS, 8>(a, n_rows, s);
+}
+
 template <typename TC>
 __global__ void __launch_bounds__(kThreads)
 embed_pos_norm_kernel(float *__restrict__ x, TC *__restrict__ copy, const void *__restrict__ table, int table_dtype,
@@ -140,8 +249,19 @@ extern "C" int sb_norm_add(float *x, void *copy, int copy_dtype, const float *pa
   const AddArgs a{x, copy, part, n_slices, slice_stride, row_stride, part_w, part_w_stride, extra, extra_w, extra_w_stride,
                   w, w_dtype, width, eps, offset, do_norm};
   hipStream_t s = (hipStream_t)stream;
+  const bool bf = copy && copy_dtype == SB_BF16;
+  const auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (width % 4 == 0 && n_slices <= kMaxFastSlices && slice_stride % 4 == 0 && row_stride % 4 == 0 && aligned(x) &&
+      aligned(part) && aligned(extra) && aligned(copy)) {
+    // (float32 throughout keeps one block shape whatever the number of rows: the order of a row's sum
+    // of squares, and so its bits, must not depend on what else the step holds)
+    bool done;
+    if (bf && n_rows <= 64) done = launch_fast<bf16_t, 1024>(a, n_rows, s);
+    else done = bf ? launch_fast<bf16_t, 256>(a, n_rows, s) : launch_fast<float, 256>(a, n_rows, s);
+    if (done) return sb::check_launch("sb_norm_add");
+  }
   const size_t lds = size_t(width) * sizeof(float);
-  if (copy && copy_dtype == SB_BF16) norm_add_kernel<bf16_t><<<n_rows, kThreads, lds, s>>>(a);
+  if (bf) norm_add_kernel<bf16_t><<<n_rows, kThreads, lds, s>>>(a);
   else norm_add_kernel<float><<<n_rows, kThreads, lds, s>>>(a);
   return sb::check_launch("sb_norm_add");
 }
