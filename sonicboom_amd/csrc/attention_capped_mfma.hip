@@ -49,6 +49,7 @@ constexpr int kValChunks = SB_PAGE * DV / 8;
 constexpr int kKeyLoads = (kKeyChunks + kThreads - 1) / kThreads;
 constexpr int kValLoads = (kValChunks + kThreads - 1) / kThreads;
 constexpr int kTile = 16;
+constexpr int kPagesInLds = 2048;           // page numbers of a block's stretch that are looked up ahead (131,072 keys)
 
 struct Args {
   bf16_t *out;                 // [rows, heads_q * DV], or NULL when partial results are written
@@ -74,6 +75,7 @@ __device__ __forceinline__ float capped(float s, float cap, float two_log2e_over
 __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   __shared__ uint4 k_lds[kKeyChunks];
   __shared__ uint4 v_lds[kValChunks];
+  __shared__ int page_lds[kPagesInLds];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
   const int group = a.heads_q / a.heads_kv, zgroups = (group + NW - 1) / NW;
   const int kvh = blockIdx.y / zgroups, hz = blockIdx.y % zgroups;
@@ -115,47 +117,66 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   floatx4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-  const float cap_arg = a.softcap > 0.0f ? 2.0f * kLog2e / a.softcap : 0.0f;
+  const float cap_arg = a.softcap > 0.0f ? a.scale * 2.0f * kLog2e / a.softcap : 0.0f;      // the scale rides along
   // scores are kept times log2(e), so that the weights are powers of two: the sink's score stays 0
   const float scale2 = a.scale * kLog2e, cap2 = a.softcap * kLog2e;
 
-  uint4 kreg[kKeyLoads], vreg[kValLoads];
-  auto fetch = [&](int c) {
-    int page = (c >= 0 && c < a.max_pages) ? table[c] : -1;
-    if (page >= a.n_pages) page = -1;
+  // two pages' loads are in flight while a third is attended (a CU holds few of these blocks: a page's
+  // round trip to memory would otherwise show once per page)
+  uint4 kreg[2][kKeyLoads], vreg[2][kValLoads];
+  // The block's page numbers go into LDS first: a look-up in memory inside the loop would have every
+  // fetch wait for the loads of the page before it (the memory counter runs in order), and the two
+  // pages in flight would be one.
+  const int n_block_pages = page_hi - page_lo + 1;
+  const bool pages_in_lds = n_block_pages <= kPagesInLds;
+  if (pages_in_lds) {
+    for (int i = tid; i < n_block_pages; i += kThreads) {
+      const int c = page_lo + i;
+      int page = (c >= 0 && c < a.max_pages) ? table[c] : -1;
+      page_lds[i] = page >= a.n_pages ? -1 : page;
+    }
+    __syncthreads();
+  }
+  auto fetch = [&](uint4 *kr, uint4 *vr, int c) {
+    int page;
+    if (pages_in_lds) {
+      page = page_lds[c - page_lo];
+    } else {
+      page = (c >= 0 && c < a.max_pages) ? table[c] : -1;
+      if (page >= a.n_pages) page = -1;
+    }
     const uint4 *kp = reinterpret_cast<const uint4 *>(a.k_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DK);
     const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DV);
 #pragma unroll
     for (int i = 0; i < kKeyLoads; ++i) {
       const int idx = tid + i * kThreads;
-      kreg[i] = (page >= 0 && idx < kKeyChunks) ? kp[idx] : make_uint4(0u, 0u, 0u, 0u);
+      kr[i] = (page >= 0 && idx < kKeyChunks) ? kp[idx] : make_uint4(0u, 0u, 0u, 0u);
     }
 #pragma unroll
     for (int i = 0; i < kValLoads; ++i) {
       const int idx = tid + i * kThreads;
-      vreg[i] = (page >= 0 && idx < kValChunks) ? vp[idx] : make_uint4(0u, 0u, 0u, 0u);
+      vr[i] = (page >= 0 && idx < kValChunks) ? vp[idx] : make_uint4(0u, 0u, 0u, 0u);
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const uint4 *kr, const uint4 *vr) {
 #pragma unroll
     for (int i = 0; i < kKeyLoads; ++i) {
       const int idx = tid + i * kThreads;
-      if (idx < kKeyChunks) k_lds[idx] = kreg[i];
+      if (idx < kKeyChunks) k_lds[idx] = kr[i];
     }
 #pragma unroll
     for (int i = 0; i < kValLoads; ++i) {
       const int idx = tid + i * kThreads;
-      if (idx < kValChunks) v_lds[idx] = vreg[i];
+      if (idx < kValChunks) v_lds[idx] = vr[i];
     }
   };
 
-  if (page_lo <= page_hi) fetch(page_lo);
-  for (int c = page_lo; c <= page_hi; ++c) {
+  auto attend = [&](uint4 *kr, uint4 *vr, int c) {
     __syncthreads();            // the page before has been read by every wave
-    stage();
+    stage(kr, vr);
     __syncthreads();
-    if (c < page_hi) fetch(c + 1);
-    if (!has_head) continue;
+    if (c + 2 <= page_hi) fetch(kr, vr, c + 2);
+    if (!has_head) return;
     const bf16_t *kl = reinterpret_cast<const bf16_t *>(k_lds);
     const bf16_t *vl = reinterpret_cast<const bf16_t *>(v_lds);
 #pragma unroll
@@ -164,43 +185,62 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
       if (first > p_last || first + 31 < lo) continue;  // uniform over the block
       // every row of the tile sees every key of this half page: no score needs a test (uniform)
       const bool whole = nr == kTile && first + 31 <= p0 && (a.window == 0 || first >= p_last - a.window + 1);
-      floatx4_t s[2];
+      // every fragment of the half page is asked of LDS before the first product: the keys' for the
+      // scores, and the values' too, which arrive while the softmax is worked out (read one by one
+      // before its product, each fragment's trip through LDS showed in full: a CU holds few waves here)
+      uint4 kf[2][KSTEPS], vf[DT];
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
         const int slot = 32 * hp + 8 * (col >> 2) + 4 * t + (col & 3);
 #pragma unroll
         for (int kc = 0; kc < KSTEPS; ++kc) {
           const int d = 32 * kc + 8 * g;
-          uint4 kf = make_uint4(0u, 0u, 0u, 0u);
-          if (d < DK) kf = *reinterpret_cast<const uint4 *>(kl + sb_key_index(slot, d, DK));
-          s[t] = mfma16(as_bf16x8(kf), qf[kc], s[t]);
+          kf[t][kc] = d < DK ? *reinterpret_cast<const uint4 *>(kl + sb_key_index(slot, d, DK)) : make_uint4(0u, 0u, 0u, 0u);
         }
       }
-      // the lane's eight scores: keys first + 8 g + 4 t + i of query column `col`
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        vf[dt] = *reinterpret_cast<const uint4 *>(vl + sb_value_index(16 * dt + col, 32 * hp + 8 * g));
+      floatx4_t s[2] = {floatx4_t{0.f, 0.f, 0.f, 0.f}, floatx4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int kc = 0; kc < KSTEPS; ++kc)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) s[t] = mfma16(as_bf16x8(kf[t][kc]), qf[kc], s[t]);      // the two tiles in turn
+      // the lane's eight scores: keys first + 8 g + 4 t + i of query column `col`, times log2(e)
       float sc[8];
       float mx = neg_inf;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int j = first + 8 * g + 4 * t + i;
           float v;
-          if (a.softcap > 0.0f) v = capped(s[t][i] * a.scale, cap2, cap_arg);
+          if (a.softcap > 0.0f) v = capped(s[t][i], cap2, cap_arg);
           else v = s[t][i] * scale2;
-          const bool visible = whole || (col < nr && j <= q_pos && j >= q_lo);
-          v = visible ? v : neg_inf;
           sc[4 * t + i] = v;
-          mx = fmaxf(mx, v);
         }
+      if (!whole) {           // uniform over the block: only pages on the diagonal or at a window's edge test their scores
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int j = first + 8 * g + e;
+          const bool visible = col < nr && j <= q_pos && j >= q_lo;
+          sc[e] = visible ? sc[e] : neg_inf;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, sc[e]);
       mx = max_over_lane_groups(mx);
       const float m_new = fmaxf(m, mx);
       const float alpha = m == neg_inf ? 0.0f : __builtin_amdgcn_exp2f(m - m_new);
       float psum = 0.0f, p[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = sc[e] == neg_inf ? 0.0f : __builtin_amdgcn_exp2f(sc[e] - m_new);
+        p[e] = __builtin_amdgcn_exp2f(sc[e] - m_new);      // 2^(-inf) is 0: a hidden key, or a row that has seen none yet
         psum += p[e];
+      }
+      if (m_new == neg_inf) {                               // (-inf) - (-inf) is no number
+        psum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p[e] = 0.0f;
       }
       l = l * alpha + psum;
       m = m_new;
@@ -208,15 +248,22 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
       pw.x = pack_bf16(p[0], p[1]); pw.y = pack_bf16(p[2], p[3]);
       pw.z = pack_bf16(p[4], p[5]); pw.w = pack_bf16(p[6], p[7]);
       const bf16x8_t pf = as_bf16x8(pw);
+      // the results so far shrink only when some row's maximum has moved (uniform over the wave)
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int d = 16 * dt + col;
-        const uint4 vf = *reinterpret_cast<const uint4 *>(vl + sb_value_index(d, 32 * hp + 8 * g));
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
-        o[dt] = mfma16(as_bf16x8(vf), pf, o[dt]);
+          for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
       }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt] = mfma16(as_bf16x8(vf[dt]), pf, o[dt]);
     }
+  };
+  if (page_lo <= page_hi) fetch(kreg[0], vreg[0], page_lo);
+  if (page_lo + 1 <= page_hi) fetch(kreg[1], vreg[1], page_lo + 1);
+  for (int c = page_lo; c <= page_hi; c += 2) {
+    attend(kreg[0], vreg[0], c);
+    if (c + 1 <= page_hi) attend(kreg[1], vreg[1], c + 1);
   }
 
   // the column's sum over the four lane groups
@@ -247,22 +294,43 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   }
 }
 
-// out[row][h][:] = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M), M the largest m_c: a thread a number
+// out[row][h][:] = sum_c o_c exp(m_c - M) / sum_c l_c exp(m_c - M), M the largest m_c: a thread a number.
+// Up to kMergeAtOnce chunks have their maxima, sums and results asked for before anything is added
+// (chunks past the last read the last again and count nothing); more chunks go in rounds of as many.
+constexpr int kMergeAtOnce = 16;
+
 __global__ void __launch_bounds__(256)
 merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml, int chunks,
              size_t n_heads /* rows * heads_q */) {
   const size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= n_heads * DV) return;
   const size_t rh = idx / DV;
-  float big = -__builtin_inff();
-  for (int c = 0; c < chunks; ++c) big = fmaxf(big, part_ml[(size_t(c) * n_heads + rh) * 2]);
+  const float neg_inf = -__builtin_inff();
+  float big = neg_inf;
+  for (int c0 = 0; c0 < chunks; c0 += kMergeAtOnce) {
+    float mc[kMergeAtOnce];
+#pragma unroll
+    for (int i = 0; i < kMergeAtOnce; ++i) mc[i] = part_ml[(size_t(min(c0 + i, chunks - 1)) * n_heads + rh) * 2];
+#pragma unroll
+    for (int i = 0; i < kMergeAtOnce; ++i) big = fmaxf(big, mc[i]);
+  }
   float num = 0.0f, den = 0.0f;
-  for (int c = 0; c < chunks; ++c) {
-    const float mc = part_ml[(size_t(c) * n_heads + rh) * 2];
-    if (mc == -__builtin_inff()) continue;
-    const float w = __builtin_amdgcn_exp2f(mc - big);          // the maxima are kept times log2(e)
-    num = fmaf(w, part_o[size_t(c) * n_heads * DV + idx], num);
-    den = fmaf(w, part_ml[(size_t(c) * n_heads + rh) * 2 + 1], den);
+  for (int c0 = 0; c0 < chunks; c0 += kMergeAtOnce) {
+    float mc[kMergeAtOnce], lc[kMergeAtOnce], oc[kMergeAtOnce];
+#pragma unroll
+    for (int i = 0; i < kMergeAtOnce; ++i) {
+      const size_t c = size_t(min(c0 + i, chunks - 1));
+      mc[i] = part_ml[(c * n_heads + rh) * 2];
+      lc[i] = part_ml[(c * n_heads + rh) * 2 + 1];
+      oc[i] = part_o[c * n_heads * DV + idx];
+    }
+#pragma unroll
+    for (int i = 0; i < kMergeAtOnce; ++i) {
+      if (c0 + i >= chunks || mc[i] == neg_inf) continue;
+      const float w = __builtin_amdgcn_exp2f(mc[i] - big);          // the maxima are kept times log2(e)
+      num = fmaf(w, oc[i], num);
+      den = fmaf(w, lc[i], den);
+    }
   }
   out[idx] = f32_to_bf16(den > 0.0f ? num / den : 0.0f);
 }

@@ -95,6 +95,65 @@ __global__ void __launch_bounds__(THREADS) headnorm_kv_store_kernel(Args a) {
   }
 }
 
+// The same for long steps of bfloat16 queries and cache, one slice, head sizes in eights: eight lanes
+// a head (more for heads above 64 numbers), eight numbers a lane in two 16-byte loads and one 16-byte store;
+// sums of squares in double by a butterfly over the head's lanes.  The arithmetic of every number is
+// that of the form above.
+template <int LANES>      // lanes a head: 8, 16 or 32 (heads of up to 64, 128, 256 numbers)
+__global__ void __launch_bounds__(256) headnorm_kv_store_wide_kernel(Args a) {
+  constexpr int HEADS_PER_BLOCK = 256 / LANES;
+  const int row = blockIdx.x, tid = threadIdx.x, sub = tid % LANES, slot_in_block = tid / LANES;
+  const float *src = a.qkv + size_t(row) * a.row_stride;
+  int page = -1, slot = 0;
+  if (a.store) {
+    const int pos = a.row_pos[row], c = pos / SB_PAGE;
+    slot = pos % SB_PAGE;
+    if (c < a.max_pages) page = a.page_table[size_t(a.row_seq[row]) * a.max_pages + c];
+    if (page >= a.n_pages) page = -1;
+  }
+  const int units = a.heads_q + (a.store ? a.heads_kv : 0);
+  for (int u0 = 0; u0 < units; u0 += HEADS_PER_BLOCK) {       // every lane walks the loop: the butterflies need them all
+    const int u = u0 + slot_in_block, d = 8 * sub;
+    const bool live = u < units && d < a.dk;
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (live) {
+      const float4 lo = *reinterpret_cast<const float4 *>(src + u * a.dk + d), hi = *reinterpret_cast<const float4 *>(src + u * a.dk + d + 4);
+      v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    }
+    double sq = 0.0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sq += double(v[i] * v[i]);
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+    if (!live) continue;
+    const bool is_q = u < a.heads_q;
+    const void *w = is_q ? a.q_w : a.k_w;
+    const float inv = w ? 1.0f / sqrtf(float(sq / double(a.dk)) + a.eps) : 1.0f;
+    uint32_t packed[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float o0 = w ? (v[2 * i] * inv) * ld_dyn(w, a.w_dtype, d + 2 * i) : v[2 * i];
+      const float o1 = w ? (v[2 * i + 1] * inv) * ld_dyn(w, a.w_dtype, d + 2 * i + 1) : v[2 * i + 1];
+      packed[i] = uint32_t(f32_to_bf16(o0)) | uint32_t(f32_to_bf16(o1)) << 16;
+    }
+    const uint4 out = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    if (is_q) *reinterpret_cast<uint4 *>((bf16_t *)a.q_out + size_t(row) * a.heads_q * a.dk + u * a.dk + d) = out;
+    else if (page >= 0)       // eight neighbouring numbers of a key stay neighbours in the cache's order
+      *reinterpret_cast<uint4 *>((bf16_t *)a.k_cache + (size_t(page) * a.heads_kv + (u - a.heads_q)) * SB_PAGE * a.dk +
+                                 sb_key_index(slot, d, a.dk)) = out;
+  }
+  if (!a.store) return;
+  const int v0 = (a.heads_q + a.heads_kv) * a.dk, nv = a.heads_kv * a.dv;
+  const float lam = a.v_first ? ld_dyn(a.lam, a.lam_dtype, 0) : 0.0f;
+  for (int e = tid; e < nv; e += 256) {
+    float v = src[v0 + e];
+    if (a.v_out) a.v_out[size_t(row) * nv + e] = v;
+    if (a.v_first) v = (1.0f - lam) * v + lam * a.v_first[size_t(row) * nv + e];
+    if (page >= 0)
+      st_f((bf16_t *)a.v_cache, (size_t(page) * a.heads_kv + e / a.dv) * a.dv * SB_PAGE + sb_value_index(e % a.dv, slot), v);
+  }
+}
+
 }  // namespace
 
 extern "C" int sb_headnorm_kv_store(void *q_out, int q_dtype, const float *qkv, int row_stride, int n_slices,
@@ -123,6 +182,12 @@ extern "C" int sb_headnorm_kv_store(void *q_out, int q_dtype, const float *qkv, 
   else if (qf) headnorm_kv_store_kernel<float, bf16_t, 256><<<n_rows, 256, 0, s>>>(a);
   else if (cf && store) headnorm_kv_store_kernel<bf16_t, float, 256><<<n_rows, 256, 0, s>>>(a);
   else if (n_rows <= 64) headnorm_kv_store_kernel<bf16_t, bf16_t, 1024><<<n_rows, 1024, 0, s>>>(a);
+  else if (n_rows >= 512 && n_slices == 1 && dk % 8 == 0 && row_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
+           (reinterpret_cast<uintptr_t>(q_out) & 15) == 0 && (!store || (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0)) {
+    if (dk <= 64) headnorm_kv_store_wide_kernel<8><<<n_rows, 256, 0, s>>>(a);
+    else if (dk <= 128) headnorm_kv_store_wide_kernel<16><<<n_rows, 256, 0, s>>>(a);
+    else headnorm_kv_store_wide_kernel<32><<<n_rows, 256, 0, s>>>(a);
+  }
   else headnorm_kv_store_kernel<bf16_t, bf16_t, 256><<<n_rows, 256, 0, s>>>(a);
   return sb::check_launch("sb_headnorm_kv_store");
 }

@@ -540,14 +540,15 @@ def test_mixed_values_are_what_the_cache_keeps(dtype):
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(4, 1, 32, 16), (6, 2, 64, 64), (16, 2, 128, 64), (5, 5, 16, 48), (9, 1, 48, 32)])
 def test_matrix_core_attention_equals_the_plain_kernel(heads, kv_heads, dim, vdim):
     """bfloat16: a prompt, portions and single rows over several pages (the pages of a step of few rows
-    are shared out over blocks and merged) against the kernel of one wave per (row, head)."""
-    n = 330
+    are shared out over blocks and merged) against the kernel of one wave per (row, head).  The steps of
+    700 and 560 rows also take the head norms' form for long steps (eight numbers a lane)."""
+    n = 700
     h = rand(n, 64).to(BF16)
     outs = {}
     for fast in (True, False):
         mixer, rt, ref, mx = attention_mixer("bfloat16", heads, kv_heads, dim, vdim, 2.0 / np.sqrt(dim), 10.0, fast=fast)
         feed = mixer_harness(mixer, rt)
-        outs[fast] = [feed(h, cuts) for cuts in ([n], [200, 17, 3] + [1] * 110)]
+        outs[fast] = [feed(h, cuts) for cuts in ([n], [560, 17, 3] + [1] * 120)]
     want, _ = T.attention(mx, 1e-5, ref, "a.", h.float().numpy())
     for a, b in zip(outs[True], outs[False]):
         part_close(a, b.float().cpu().numpy(), "bfloat16", "matrix cores against the plain kernel", bf16=1.5e-2)
