@@ -69,7 +69,8 @@ typedef enum sb_status {
 
 typedef enum sb_dtype { SB_F32 = 0, SB_BF16 = 1 } sb_dtype;
 
-/* The `gated` argument of the products and of sb_gate_mul: not gated, or the activation of the
+/* The `gated` argument of the products and of sb_gate_mul: not gated, or the activation (SiLU, the tanh
+ * form of GELU, max(g, 0)) of the
  * gate in Y = act(X Wg^T) * (X Wu^T). */
 typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2, SB_GATE_RELU = 3 } sb_gate;
 
@@ -229,6 +230,76 @@ int sb_latent_attention_bf16(void *out, const void *q, const void *cache, const 
                              int max_pages, int n_pages_total, const int32_t *row_pos, const int32_t *tiles,
                              int n_tiles, int heads, int rank, int rot_dim, float scale, int window,
                              int tile_rows, int n_splits, float *part_o, float *part_ml, int n_rows, void *stream);
+
+/* ---- norms on what a sublayer gives back, an embedding with positions (csrc/outnorm.hip) --------
+ * un(v) = v / sqrt(mean(v^2) + eps) * (offset + w): offset 1 for weights kept as multiplier minus one.
+ * sb_offset_norm: y[r,:] = un(x[rows ? rows[r] : r,:]).
+ * sb_norm_add: x[t,:] += un(sum_s a_s(t) part[s * slice_stride + t * row_stride + :] (+ b(t) extra[t,:])),
+ *   a_s(t) = part_w ? part_w[t * part_w_stride + s] : 1, b(t) = extra_w ? extra_w[t * extra_w_stride] : 1;
+ *   do_norm 0: the sum is added as it is; copy (NULL or of copy_dtype): the new x.
+ * sb_embed_pos_norm: x[r,:] = table[ids[r],:] * scale (+ pos_table[row_pos[r],:]), normed with do_norm; an id
+ *   or a position outside its table gives a row of NaN. */
+int sb_offset_norm(void *y, int out_dtype, const float *x, const void *w, int w_dtype, const int32_t *rows,
+                   int n_rows, int width, float eps, float offset, void *stream);
+int sb_norm_add(float *x, void *copy, int copy_dtype, const float *part, int n_slices, size_t slice_stride,
+                size_t row_stride, const float *part_w, int part_w_stride, const float *extra,
+                const float *extra_w, int extra_w_stride, const void *w, int w_dtype, int n_rows, int width,
+                float eps, float offset, int do_norm, void *stream);
+int sb_embed_pos_norm(float *x, void *copy, int copy_dtype, const void *table, int table_dtype,
+                      const void *pos_table, int pos_dtype, const int32_t *ids, const int32_t *row_pos,
+                      int n_rows, int vocab, int n_positions, float scale, const void *w, int w_dtype,
+                      int width, float eps, float offset, int do_norm, void *stream);
+/* x[i] *= scale. */
+int sb_scale(float *x, float scale, size_t n, void *stream);
+
+/* ---- head norms, value mixing and store (csrc/headnorm_kv.hip) ---------------------------------
+ * qkv f32 [n_slices][n_rows][row_stride] = [q: heads_q x dk | k: heads_kv x dk | v: heads_kv x dv], slices
+ * added in ascending order; every head of q and k divided by its root mean square (eps inside the root)
+ * times q_w / k_w [dk] (NULL: as it is); v <- (1 - lam) v + lam v_first when v_first is given; the v of
+ * before the mixing to v_out when that is given; q out in q_dtype, k and v (store != 0) into the pages. */
+int sb_headnorm_kv_store(void *q_out, int q_dtype, const float *qkv, int row_stride, int n_slices,
+                         const void *q_w, const void *k_w, int w_dtype, float eps, const float *v_first,
+                         const void *lam, int lam_dtype, float *v_out, const int32_t *row_pos,
+                         const int32_t *row_seq, void *k_cache, void *v_cache, int cache_dtype,
+                         const int32_t *page_table, int max_pages, int n_pages, int n_rows, int heads_q,
+                         int heads_kv, int dk, int dv, int store, void *stream);
+
+/* sb_attention with values of v_dim numbers a head (cache values [page][kv head][v_dim][position], out
+ * [rows, heads_q * v_dim]), scores capped as softcap * tanh(s / softcap) when softcap > 0, and with `sink`
+ * one more key of score 0 without a value in every softmax. */
+int sb_attention_capped(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                        const void *v_cache, int cache_dtype, const int32_t *page_table, int max_pages,
+                        int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows,
+                        int heads_q, int heads_kv, int head_dim, int v_dim, float scale, int window,
+                        float softcap, int sink, void *stream);
+
+/* ---- routed experts (csrc/moe.hip, csrc/moe_mfma.hip) -------------------------------------------
+ * sb_moe_route: from scores z f32 [rows, stride] the `top` largest of the first n_experts (ties to the
+ *   lower number) in falling order, ids int32 [rows, top], and weights f32 [rows, top + 1]: the softmax
+ *   over the chosen scores, then sigmoid(z[n_experts]) with has_gate (else 0).
+ * sb_moe_router: the same from z = h w^T, w f32 [n_experts (+ 1), n_in], h of h_dtype, in one launch.
+ * sb_moe_product: Y[p,:] = X[p / x_div,:] W_e^T, e = ids[p] (NULL: expert 0), W [experts][out (x 2 gated)][in];
+ *   gated: g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = u cut to +-limit.  Plain kernel, any sizes.
+ * sb_moe_group / sb_moe_product_bf16: the pairs laid out expert by expert on the device (order, tiles of
+ *   tile_rows = sb_moe_tile_rows(pairs, experts) pairs, their count) and the product on the matrix cores.
+ * sb_swish_clamp_mul: the gated pair of gu f32 [rows, 2 * width]. */
+int sb_moe_max_top(void);
+int sb_moe_route(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                 int top, int has_gate, void *stream);
+int sb_moe_router(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                  int n_in, int n_experts, int top, int has_gate, void *stream);
+int sb_moe_product(void *y, int y_dtype, const void *x, int x_dtype, const void *w, int w_dtype,
+                   const int32_t *ids, int n_pairs, int x_div, int n_out, int n_in, int n_experts,
+                   int gated, float limit, float alpha, void *stream);
+int sb_moe_tile_rows(int n_pairs, int n_experts);
+int sb_moe_group(const int32_t *ids, int n_pairs, int n_experts, int tile_rows, int32_t *order, int32_t *tiles,
+                 int32_t *n_tiles, void *stream);
+int sb_moe_product_bf16_ok(int n_in);
+int sb_moe_product_bf16(void *y, int y_dtype, const void *x, const void *w, const int32_t *order,
+                        const int32_t *tiles, const int32_t *n_tiles, int max_tiles, int tile_rows, int n_pairs,
+                        int x_div, int n_out, int n_in, int gated, float limit, float alpha, void *stream);
+int sb_swish_clamp_mul(void *out, int out_dtype, const float *gu, int n_rows, int width, float limit, float alpha,
+                       void *stream);
 
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts

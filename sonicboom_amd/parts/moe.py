@@ -8,10 +8,12 @@
     u' = W_up f cut to [-limit, limit]                                  ("swish_clamp")
 
 The router runs in float32 whatever the model's type (its matrix, with the shared expert's gate
-row under it, is kept in float32; one kernel makes the scores and the choice).  Choice and weights are made on the
-device, and the experts' products find their rows there too: nothing of a step depends on a value the
-host has seen, so a decode step can be recorded and replayed.  The experts' matrices are stacked
-when the part is built: [experts, 2 * inner, width] (gate over up) and [experts, width, inner].
+row under it, is kept in float32; one kernel makes the scores and the choice).  Choice and weights
+are made on the device, and the experts' products find their rows there too: nothing of a step
+depends on a value the host has seen, so a decode step can be recorded and replayed.  The experts'
+matrices are stacked when the part is built: [experts, 2 * inner, width] (gate over up) and
+[experts, width, inner].  The expert that every row takes is a dense feed-forward: its two products
+are the framework's own, with the clamped pair applied to the float32 result of the stacked one.
 
 Every (row, choice) pair has its own row of the intermediate and of the result; the pass that
 ends the sublayer adds a row's pairs in the order of the choice, times their weights.  A pair's
